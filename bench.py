@@ -1,0 +1,197 @@
+"""Throughput of the ragged_dot hot path on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+
+One step = one pass of the hot path over one synthetic batch already resident in HBM: forward for the forward-only
+workloads, forward + dlhs + drhs for the others.  Prints one JSON line (see the keys below).  The default workload is
+the Mixtral-8x7B-shaped forward+backward.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2516.6  # dense bf16 MFMA: 256 CU x 4 SIMD x 1024 FLOP/clk x 2.4 GHz
+PEAK_HBM_GBS = 8000.0
+
+
+def _event_ms(fn, reps, torch):
+    """Average milliseconds per call of fn() over `reps` back-to-back calls, by events on the launch stream."""
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(reps):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / reps
+
+
+def cpu_baseline(name, seconds_hint=20.0):
+    """The numpy oracle on this host's cores, on a bounded sample of the same workload: whole groups (all their rows,
+    the full k and n), forward (+ backward where the workload has one), until about `seconds_hint` of work is done."""
+    import numpy as np
+
+    from gpu_ragged_dot_amd import workloads
+    from oracle import ragged_dot_oracle as oracle
+
+    w = workloads.WORKLOADS[name]
+    gs = workloads.group_sizes(name)
+    order = [i for i in np.argsort(-gs) if gs[i] > 0]
+    rng = np.random.default_rng(0)
+    done_flops, done_bytes, elapsed, used = 0.0, 0.0, 0.0, []
+    for gi in order:
+        rows = int(gs[gi])
+        x = oracle.round_to(rng.standard_normal((rows, w.k), dtype=np.float32), "bfloat16")
+        A = oracle.round_to(rng.standard_normal((1, w.k, w.n), dtype=np.float32) / np.sqrt(w.k), "bfloat16")
+        one = np.array([rows], np.int32)
+        t0 = time.perf_counter()
+        oracle.gmm(x, A, one)
+        if w.backward:
+            dout = x[:, :1] * np.ones((1, w.n), np.float32)
+            oracle.gmm_vjp(x, A, one, dout)
+        elapsed += time.perf_counter() - t0
+        done_flops += 2.0 * rows * w.k * w.n * (3 if w.backward else 1)
+        done_bytes += w.k * w.n * 2
+        used.append(int(gi))
+        if elapsed >= seconds_hint or len(used) >= 64:
+            break
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    if name == "decode":
+        value, unit = done_bytes / elapsed / 1e9, "GB/s"
+    else:
+        value, unit = done_flops / elapsed / 1e12, "TFLOP/s"
+    return {
+        "value": value,
+        "unit": unit,
+        "cores": cores,
+        "kind": "port",
+        "sample": f"numpy oracle (fp32 BLAS per group) on {len(used)} whole group(s) of '{name}' "
+                  f"({sum(int(gs[i]) for i in used)} rows), {elapsed:.1f} s",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="mixtral_fwd_bwd")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py measures one GPU: the ragged_dot path has no multi-GPU part; run with --gpus 1")
+
+    import torch
+
+    import gpu_ragged_dot_amd as rd
+    from gpu_ragged_dot_amd import _capi, ops, planner, workloads
+
+    name = args.workload
+    w = workloads.WORKLOADS[name]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    x, A, dout, gs = workloads.make_inputs(name, device=dev)
+    hp = dict(block_m=64, block_k=64, block_n=64, interpret=False, compute_dtype=None, acc_dtype=torch.float32, chunk_m=512)
+
+    # For the memory-bound decode shape the 167 MB of expert weights would otherwise sit in the 256 MB last-level
+    # cache between steps: rotate over several copies so that every step streams from HBM.
+    copies = [A]
+    if name == "decode":
+        copies = [A] + [A.clone() for _ in range(5)]
+    state = {"i": 0}
+
+    def fwd():
+        a = copies[state["i"] % len(copies)]
+        state["i"] += 1
+        return ops._gmm_fwd(x, a, gs, **hp, trans_rhs=False)
+
+    def dlhs():
+        return ops._gmm_fwd(dout, A, gs, **hp, trans_rhs=True)
+
+    def drhs():
+        return ops._tgmm_fwd(x, dout, gs, **hp)
+
+    parts = [("fwd", fwd)] + ([("dlhs", dlhs), ("drhs", drhs)] if w.backward else [])
+
+    def step():
+        for _, fn in parts:
+            fn()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ms_per_step = _event_ms(step, args.steps, torch)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    # per-kernel launch durations, for the roofline of the dominant kernel
+    per = {pname: _event_ms(fn, max(args.steps, 5), torch) for pname, fn in parts}
+    dominant = max(per, key=per.get)
+    flops_step = workloads.flops(name)
+    abytes = workloads.algorithmic_bytes(name)
+    flops_one = flops_step / (3 if w.backward else 1)
+
+    if name == "decode":
+        metric, unit = "ragged_dot decode forward, expert weights streamed", "GB/s"
+        value = abytes["weights_read"] / (ms_per_step * 1e-3) / 1e9
+        roof = {"bound": "hbm", "achieved": abytes[dominant] / (per[dominant] * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                "unit": "GB/s"}
+    else:
+        metric, unit = ("ragged_dot fwd+bwd" if w.backward else "ragged_dot fwd") + " throughput", "TFLOP/s"
+        value = flops_step / (ms_per_step * 1e-3) / 1e12
+        t_flop = flops_one / (PEAK_BF16_TFLOPS * 1e12)
+        t_byte = abytes[dominant] / (PEAK_HBM_GBS * 1e9)
+        if t_byte > t_flop:
+            roof = {"bound": "hbm", "achieved": abytes[dominant] / (per[dominant] * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                    "unit": "GB/s"}
+        else:
+            roof = {"bound": "mfma", "achieved": flops_one / (per[dominant] * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
+                    "unit": "TFLOP/s"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = None
+    roof["kernel"] = {"fwd": "gmm_kernel (NN)" if name != "decode" else "gmm_decode_kernel", "dlhs": "gmm_kernel (NT)",
+                      "drhs": "tgmm_kernel"}[dominant]
+    roof["launch_ms"] = per[dominant]
+
+    plans = {}
+    for pname, op, (mm, kk, nn) in (("fwd", 0, (w.m, w.k, w.n)), ("dlhs", 1, (w.m, w.n, w.k)), ("drhs", 2, (w.m, w.k, w.n))):
+        if pname in per:
+            p = planner.select_plan(op, mm, kk, nn, w.g)
+            plans[pname] = ("decode_nb%d" % p.decode_nb) if p.decode_nb else planner.compiled_variants()[p.variant].name.decode()
+
+    out = {
+        "metric": metric,
+        "value": value,
+        "unit": unit,
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": name, "m": w.m, "k": w.k, "n": w.n, "g": w.g, "backward": w.backward,
+                   "description": w.description, "group_sizes": "seeded, see gpu_ragged_dot_amd/workloads.py"},
+        "frac_of_bf16_mfma_peak": (value / PEAK_BF16_TFLOPS) if unit == "TFLOP/s" else None,
+        "per_kernel_ms": per,
+        "tile_plans": plans,
+        "wall_s_timed_region": wall,
+        "roofline": roof,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(name, args.cpu_seconds)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

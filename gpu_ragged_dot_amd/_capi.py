@@ -1,0 +1,126 @@
+"""ctypes binding of ``csrc/libragged_dot_hip.so`` (the C ABI declared in ``include/ragged_dot_hip.h``).
+
+The library is built in-tree by ``make -C gpu_ragged_dot_amd/csrc`` (or ``__graft_entry__.build()``).  There is no
+fallback: if the shared object is missing, importing this module raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch  # noqa: F401  - loaded first so the HIP runtime already in the process is the one the library binds to
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libragged_dot_hip.so")
+
+RD_DTYPE_BF16 = 0
+RD_DTYPE_F32 = 1
+
+RD_OK = 0
+RD_ERR_INVALID_ARGUMENT = -1
+RD_ERR_UNSUPPORTED = -2
+RD_ERR_WORKSPACE = -3
+RD_ERR_HIP = -4
+
+OP_GMM, OP_GMM_TRANS, OP_TGMM = 0, 1, 2
+
+
+class RaggedDotError(RuntimeError):
+    """A call into the HIP library returned a non-zero status."""
+
+    def __init__(self, status: int, message: str):
+        super().__init__(f"ragged_dot_hip status {status}: {message}")
+        self.status = status
+
+
+class VariantInfo(ctypes.Structure):
+    _fields_ = [
+        ("id", ctypes.c_int),
+        ("tile_m", ctypes.c_int),
+        ("tile_n", ctypes.c_int),
+        ("tile_k", ctypes.c_int),
+        ("waves_m", ctypes.c_int),
+        ("waves_n", ctypes.c_int),
+        ("vec", ctypes.c_int),
+        ("name", ctypes.c_char * 48),
+    ]
+
+
+class Plan(ctypes.Structure):
+    _fields_ = [("variant", ctypes.c_int), ("group_m", ctypes.c_int), ("decode_nb", ctypes.c_int)]
+
+    def __repr__(self):
+        return f"Plan(variant={self.variant}, group_m={self.group_m}, decode_nb={self.decode_nb})"
+
+
+# every symbol the header declares; checked at load time
+EXPORTS = (
+    "rd_abi_version",
+    "rd_last_error",
+    "rd_num_variants",
+    "rd_get_variant",
+    "rd_default_plan",
+    "rd_sched_map",
+    "rd_sched_map_len",
+    "rd_gmm_workspace_bytes",
+    "rd_gmm",
+    "rd_tgmm_workspace_bytes",
+    "rd_tgmm",
+)
+
+
+def _load() -> ctypes.CDLL:
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `make -C {os.path.dirname(LIB_PATH)} -j8` "
+            "(hipcc --offload-arch=gfx950).  There is no CPU or PyTorch fallback for these ops."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name in EXPORTS:
+        if not hasattr(lib, name):
+            raise ImportError(f"{LIB_PATH} does not export {name}")
+    vp, ip, i, sz = ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+    lib.rd_abi_version.restype = i
+    lib.rd_last_error.restype = ctypes.c_char_p
+    lib.rd_num_variants.restype = i
+    lib.rd_get_variant.argtypes = [i, ctypes.POINTER(VariantInfo)]
+    lib.rd_get_variant.restype = i
+    lib.rd_default_plan.argtypes = [i, i, i, i, i, i, ctypes.POINTER(Plan)]
+    lib.rd_default_plan.restype = i
+    lib.rd_sched_map.argtypes = [vp, ip, i, i, i, ip, ip, ip, ip]
+    lib.rd_sched_map.restype = i
+    lib.rd_sched_map_len.argtypes = [i, i, i]
+    lib.rd_sched_map_len.restype = i
+    lib.rd_gmm_workspace_bytes.argtypes = [i, i, ctypes.POINTER(Plan)]
+    lib.rd_gmm_workspace_bytes.restype = sz
+    lib.rd_gmm.argtypes = [vp, vp, vp, ip, vp, i, i, i, i, i, i, ctypes.POINTER(Plan), vp, sz]
+    lib.rd_gmm.restype = i
+    lib.rd_tgmm_workspace_bytes.argtypes = [i, i, ctypes.POINTER(Plan)]
+    lib.rd_tgmm_workspace_bytes.restype = sz
+    lib.rd_tgmm.argtypes = [vp, vp, vp, ip, vp, i, i, i, i, i, ctypes.POINTER(Plan), vp, sz]
+    lib.rd_tgmm.restype = i
+    return lib
+
+
+lib = _load()
+
+
+def check(status: int) -> None:
+    if status != RD_OK:
+        raise RaggedDotError(status, (lib.rd_last_error() or b"").decode("utf-8", "replace"))
+
+
+def variants() -> list[VariantInfo]:
+    out = []
+    for idx in range(lib.rd_num_variants()):
+        info = VariantInfo()
+        check(lib.rd_get_variant(idx, ctypes.byref(info)))
+        out.append(info)
+    return out
+
+
+def default_plan(op: int, m: int, k: int, n: int, g: int, dtype: int = RD_DTYPE_BF16) -> Plan:
+    plan = Plan()
+    check(lib.rd_default_plan(op, m, k, n, g, dtype, ctypes.byref(plan)))
+    return plan

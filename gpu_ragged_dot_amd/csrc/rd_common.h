@@ -1,0 +1,43 @@
+// Shared device-side helpers for the ragged_dot HIP kernels (gfx950 / CDNA4 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace rd {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef short s16x8_t __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+typedef uint16_t bf16_bits;  // storage type of a bf16 element in HBM / LDS
+
+// fp32 -> bf16, round to nearest even (v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ bf16_bits f32_to_bf16(float f) {
+  __bf16 h = (__bf16)f;
+  return __builtin_bit_cast(bf16_bits, h);
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+
+__device__ __forceinline__ float bf16_to_f32(bf16_bits b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
+
+__device__ __forceinline__ int imin(int a, int b) { return a < b ? a : b; }
+__device__ __forceinline__ int imax(int a, int b) { return a > b ? a : b; }
+
+// Work-groups are dealt to the 8 XCDs round-robin by launch index.  Remap the launch index so that each XCD
+// (own 4 MB L2) walks one contiguous range of logical tile ids.  Returns -1 for the padding of the last range.
+__device__ __forceinline__ int xcd_contiguous_id(int launch_id, int n_logical) {
+  const int per_xcd = (n_logical + 7) >> 3;
+  const int id = (launch_id & 7) * per_xcd + (launch_id >> 3);
+  return id < n_logical ? id : -1;
+}
+
+static inline int xcd_padded_grid(int n_logical) { return ((n_logical + 7) / 8) * 8; }
+
+}  // namespace rd

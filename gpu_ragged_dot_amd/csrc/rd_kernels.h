@@ -1,0 +1,150 @@
+// Grouped-GEMM kernels built on gemm_tile(): launch-index -> tile mapping, group lookup through the scheduling
+// map, tail / empty-group zeroing.
+#pragma once
+#include "rd_gemm_tile.h"
+
+namespace rd {
+
+// y[m, n] = ragged x[m, k] . A[g]  (A is [g, k, n], or [g, n, k] when trans_rhs).
+struct GmmArgs {
+  const bf16_bits* x;
+  const bf16_bits* A;
+  bf16_bits* y;
+  const int32_t* group_sizes;    // [g]
+  const int32_t* group_offsets;  // [g]   exclusive prefix sum of group_sizes
+  const int32_t* tile2group;     // [U]   scheduling map built with chunk = tile height
+  const int32_t* tile2it;        // [U]
+  const int32_t* total_tiles;    // [1]
+  int m, k, n, g;
+  int U;        // static bound on row tiles: ceil(m / BM) + g
+  int n_tiles;  // ceil(n / BN)
+  int group_m;  // row tiles per band of the tile walk
+};
+
+// dA[g, k, n] = x[rows of g, k]^T . dy[rows of g, n]
+struct TgmmArgs {
+  const bf16_bits* x;
+  const bf16_bits* dy;
+  bf16_bits* dA;
+  const int32_t* group_sizes;
+  const int32_t* group_offsets;
+  int m, k, n, g;
+  int k_tiles, n_tiles;  // ceil(k / BM), ceil(n / BN)
+  int group_m;
+};
+
+// Walk tiles in bands of `group_m` rows: consecutive ids share B columns / A rows so that the ~32 tiles one XCD
+// has in flight re-use each other's operands out of its L2.
+__device__ __forceinline__ void band_walk(int id, int rows, int cols, int group_m, int& ri, int& cj) {
+  const int band_sz = group_m * cols;
+  const int band = id / band_sz;
+  const int within = id - band * band_sz;
+  const int gm = imin(group_m, rows - band * group_m);
+  cj = within / gm;
+  ri = band * group_m + (within - cj * gm);
+}
+
+template <class C, bool TRANS_RHS>
+__global__ __launch_bounds__(C::NT) void gmm_kernel(GmmArgs p) {
+  extern __shared__ __attribute__((aligned(16))) bf16_bits smem[];
+  const int id = xcd_contiguous_id(blockIdx.x, p.U * p.n_tiles);
+  if (id < 0) return;
+  int mi, nj;
+  band_walk(id, p.U, p.n_tiles, p.group_m, mi, nj);
+
+  const int total = imin(*p.total_tiles, p.U);
+  const int col0 = nj * C::BN;
+  const int cols = imin(C::BN, p.n - col0);
+
+  if (mi < total) {
+    const int gi = p.tile2group[mi];
+    const int it = p.tile2it[mi];
+    const int row0 = p.group_offsets[gi] + it * C::BM;
+    int rows = imin(C::BM, p.group_sizes[gi] - it * C::BM);
+    rows = imin(rows, p.m - row0);  // group_sizes summing past m: never touch rows >= m
+    if (rows <= 0 || row0 < 0) return;
+    const bf16_bits* Ap = p.x + (size_t)row0 * p.k;
+    const bf16_bits* Bp = TRANS_RHS ? p.A + (size_t)gi * p.n * p.k + (size_t)col0 * p.k
+                                    : p.A + (size_t)gi * p.k * p.n + col0;
+    bf16_bits* Op = p.y + (size_t)row0 * p.n + col0;
+    gemm_tile<C>(Ap, p.k, rows, Bp, TRANS_RHS ? p.k : p.n, cols, p.k, Op, p.n, smem);
+  } else {
+    // Rows past sum(group_sizes) are defined to be zero.  The map never uses more than
+    // U - ceil(tail / BM) entries, so the unused tile slots cover the tail.
+    long long s = (long long)p.group_offsets[p.g - 1] + p.group_sizes[p.g - 1];
+    if (s < 0) s = 0;
+    const long long r0 = s + (long long)(mi - total) * C::BM;
+    if (r0 >= p.m) return;
+    const int rows = imin(C::BM, p.m - (int)r0);
+    zero_tile<C::NT, C::VEC>(p.y + (size_t)r0 * p.n + col0, p.n, rows, cols);
+  }
+}
+
+template <class C>
+__global__ __launch_bounds__(C::NT) void tgmm_kernel(TgmmArgs p) {
+  extern __shared__ __attribute__((aligned(16))) bf16_bits smem[];
+  const int per_group = p.k_tiles * p.n_tiles;
+  const int id = xcd_contiguous_id(blockIdx.x, p.g * per_group);
+  if (id < 0) return;
+  const int gi = id / per_group;
+  int ri, cj;
+  band_walk(id - gi * per_group, p.k_tiles, p.n_tiles, p.group_m, ri, cj);
+
+  const int kk0 = ri * C::BM, col0 = cj * C::BN;
+  const int krows = imin(C::BM, p.k - kk0), cols = imin(C::BN, p.n - col0);
+  bf16_bits* Op = p.dA + (size_t)gi * p.k * p.n + (size_t)kk0 * p.n + col0;
+
+  const int row0 = p.group_offsets[gi];
+  int rows = p.group_sizes[gi];
+  rows = imin(rows, p.m - row0);
+  if (rows <= 0 || row0 < 0) {  // empty group: its slice of dA is zero
+    zero_tile<C::NT, C::VEC>(Op, p.n, krows, cols);
+    return;
+  }
+  const bf16_bits* Ap = p.x + (size_t)row0 * p.k + kk0;
+  const bf16_bits* Bp = p.dy + (size_t)row0 * p.n + col0;
+  gemm_tile<C>(Ap, p.k, krows, Bp, p.n, cols, rows, Op, p.n, smem);
+}
+
+// ---- host-side launchers, one set per compiled tile shape -------------------------------------------------------
+
+typedef int (*gmm_launch_fn)(hipStream_t, const GmmArgs&);
+typedef int (*tgmm_launch_fn)(hipStream_t, const TgmmArgs&);
+
+struct TileVariant {
+  const char* name;
+  int bm, bn, bk, waves_m, waves_n;
+  int vec;  // 1: needs k % 8 == 0 and n % 8 == 0 (16-byte row pitches); 0: any shape
+  gmm_launch_fn gmm_nn, gmm_nt;
+  tgmm_launch_fn tgmm;
+};
+
+// Kernels that use more than 64 KB of LDS must opt in, once per device.
+static inline int allow_big_lds(const void* kern, int bytes) {
+  if (bytes <= 64 * 1024) return hipSuccess;
+  return (int)hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
+template <class C, bool TRANS_RHS>
+int launch_gmm(hipStream_t s, const GmmArgs& a) {
+  auto kern = gmm_kernel<C, TRANS_RHS>;
+  const int attr_rc = allow_big_lds(reinterpret_cast<const void*>(kern), C::LDS_BYTES);
+  if (attr_rc != hipSuccess) return attr_rc;
+  const int grid = xcd_padded_grid(a.U * a.n_tiles);
+  if (grid <= 0) return hipSuccess;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(C::NT), C::LDS_BYTES, s, a);
+  return (int)hipGetLastError();
+}
+
+template <class C>
+int launch_tgmm(hipStream_t s, const TgmmArgs& a) {
+  auto kern = tgmm_kernel<C>;
+  const int attr_rc = allow_big_lds(reinterpret_cast<const void*>(kern), C::LDS_BYTES);
+  if (attr_rc != hipSuccess) return attr_rc;
+  const int grid = xcd_padded_grid(a.g * a.k_tiles * a.n_tiles);
+  if (grid <= 0) return hipSuccess;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(C::NT), C::LDS_BYTES, s, a);
+  return (int)hipGetLastError();
+}
+
+}  // namespace rd

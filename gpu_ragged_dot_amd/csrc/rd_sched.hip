@@ -1,0 +1,118 @@
+// group_sizes -> (tile -> group, tile -> index inside group, row offsets) scheduling map, as one prefix-sum
+// kernel.  Produces exactly the five arrays of the reference's GMMGroupLookupMetadata
+// (gpu_ragged_dot.py:60-90) in int32, every output element written once.
+#include "rd_common.h"
+#include "rd_sched.h"
+
+namespace rd {
+
+namespace {
+
+constexpr int kSchedThreads = 1024;
+constexpr int kSchedWaves = kSchedThreads / 64;
+
+// floor(a / b) for b > 0, as numpy's // on int32.
+__device__ __forceinline__ int32_t floor_div(int32_t a, int32_t b) {
+  int32_t q = a / b;
+  return (a % b != 0 && a < 0) ? q - 1 : q;
+}
+
+// Inclusive scan across the work-group of two values at once; every thread gets its inclusive sums and the
+// work-group totals.  Sums wrap like int32 cumsum does.
+__device__ __forceinline__ void block_scan2(uint32_t& a, uint32_t& b, uint32_t& total_a, uint32_t& total_b,
+                                            uint32_t* wave_a, uint32_t* wave_b) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const uint32_t ua = __shfl_up(a, d, 64), ub = __shfl_up(b, d, 64);
+    if (lane >= d) { a += ua; b += ub; }
+  }
+  if (lane == 63) { wave_a[wave] = a; wave_b[wave] = b; }
+  __syncthreads();
+  uint32_t pa = 0, pb = 0, ta = 0, tb = 0;
+#pragma unroll
+  for (int w = 0; w < kSchedWaves; ++w) {
+    const uint32_t xa = wave_a[w], xb = wave_b[w];
+    if (w < wave) { pa += xa; pb += xb; }
+    ta += xa; tb += xb;
+  }
+  a += pa; b += pb;
+  total_a = ta; total_b = tb;
+  __syncthreads();
+}
+
+__global__ __launch_bounds__(kSchedThreads) void sched_map_kernel(const int32_t* __restrict__ gs, int g, int U,
+                                                                  int chunk, int32_t* __restrict__ group_offsets,
+                                                                  int32_t* __restrict__ tile2group,
+                                                                  int32_t* __restrict__ tile2it,
+                                                                  int32_t* __restrict__ total_tiles) {
+  __shared__ uint32_t wave_a[kSchedWaves], wave_b[kSchedWaves];
+  __shared__ int32_t incl[kSchedThreads];  // inclusive tile-count scan of the current slab of groups
+  const int tid = threadIdx.x;
+  uint32_t carry_rows = 0, carry_tiles = 0;
+
+  for (int base = 0; base < g; base += kSchedThreads) {
+    const int gi = base + tid;
+    const int32_t sz = gi < g ? gs[gi] : 0;
+    const int32_t bpg = gi < g ? floor_div(sz + chunk - 1, chunk) : 0;  // gpu_ragged_dot.py:73
+    uint32_t a = (uint32_t)sz, b = (uint32_t)bpg, ta, tb;
+    block_scan2(a, b, ta, tb, wave_a, wave_b);
+    if (gi < g) group_offsets[gi] = (int32_t)(carry_rows + a - (uint32_t)sz);  // :86
+    incl[tid] = (int32_t)(carry_tiles + b);
+    __syncthreads();
+
+    // Tiles [carry_tiles, carry_tiles + tb) belong to this slab of groups (:76-82).
+    const int32_t lo = (int32_t)carry_tiles, hi = (int32_t)(carry_tiles + tb);
+    const int cnt = imin(kSchedThreads, g - base);
+    for (int32_t t = imax(lo, 0) + tid; t < hi && t < U; t += kSchedThreads) {
+      int l = 0, r = cnt;  // first j with incl[j] > t; empty groups repeat their predecessor and are skipped
+      while (l < r) {
+        const int mid = (l + r) >> 1;
+        if (incl[mid] > t) r = mid; else l = mid + 1;
+      }
+      const int32_t start = l == 0 ? lo : incl[l - 1];
+      tile2group[t] = base + l;
+      tile2it[t] = t - start;
+    }
+    carry_rows += ta;
+    carry_tiles += tb;
+    __syncthreads();
+  }
+  // Unused slots read as zero (the masked sums of :81-82 are empty there).
+  for (int32_t t = imax((int32_t)carry_tiles, 0) + tid; t < U; t += kSchedThreads) {
+    tile2group[t] = 0;
+    tile2it[t] = 0;
+  }
+  if (tid == 0) *total_tiles = (int32_t)carry_tiles;  // :89
+}
+
+template <typename T>
+__global__ void fill_kernel(T* p, size_t n, T v) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
+}
+
+}  // namespace
+
+int launch_sched_map(hipStream_t s, const int32_t* gs, int g, int m, int chunk, int32_t* group_offsets,
+                     int32_t* tile2group, int32_t* tile2it, int32_t* total_tiles) {
+  const int U = (m + chunk - 1) / chunk + g;  // gpu_ragged_dot.py:77
+  hipLaunchKernelGGL(sched_map_kernel, dim3(1), dim3(kSchedThreads), 0, s, gs, g, U, chunk, group_offsets,
+                     tile2group, tile2it, total_tiles);
+  return (int)hipGetLastError();
+}
+
+int launch_zero_bytes(hipStream_t s, void* p, size_t bytes) {
+  if (bytes == 0) return hipSuccess;
+  // Callers may be under graph capture, where memset nodes are unreliable: clear with a plain kernel.
+  if (bytes % 4 == 0 && (reinterpret_cast<uintptr_t>(p) % 4) == 0) {
+    const size_t n = bytes / 4;
+    const int grid = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+    hipLaunchKernelGGL(fill_kernel<uint32_t>, dim3(grid), dim3(256), 0, s, (uint32_t*)p, n, 0u);
+  } else {
+    const int grid = (int)((bytes + 255) / 256 < 4096 ? (bytes + 255) / 256 : 4096);
+    hipLaunchKernelGGL(fill_kernel<uint8_t>, dim3(grid), dim3(256), 0, s, (uint8_t*)p, bytes, (uint8_t)0);
+  }
+  return (int)hipGetLastError();
+}
+
+}  // namespace rd

@@ -1,0 +1,264 @@
+"""``ragged_dot`` / ``trans_ragged_dot`` with the reference's Python signature, running on HIP kernels.
+
+Mirrors gpu_ragged_dot.py:345-454 (``gmm``, ``tgmm``, their aliases and the custom VJP).  Arrays are
+``torch.Tensor`` on a ROCm device: torch supplies device memory and the stream, nothing else - every product is
+computed by ``csrc/libragged_dot_hip.so`` through its C ABI.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import _capi, planner
+from .planner import CHUNK_M, DEFAULT_BLOCK_K, DEFAULT_BLOCK_M, DEFAULT_BLOCK_N
+
+__all__ = ["gmm", "tgmm", "ragged_dot", "trans_ragged_dot", "ragged_dot_vjp", "make_group_metadata"]
+
+_DTYPES = {torch.bfloat16: _capi.RD_DTYPE_BF16, torch.float32: _capi.RD_DTYPE_F32}
+
+
+def _dtype_code(t: torch.Tensor, compute_dtype, acc_dtype) -> int:
+    if t.dtype not in _DTYPES:
+        raise TypeError(f"unsupported dtype {t.dtype}; bf16 is the compiled operand type")
+    if compute_dtype is not None and compute_dtype != t.dtype:
+        raise NotImplementedError(f"compute_dtype={compute_dtype} differs from the operand dtype {t.dtype}")
+    if acc_dtype not in (None, torch.float32):
+        raise NotImplementedError("accumulation is always float32 on the matrix cores")
+    return _DTYPES[t.dtype]
+
+
+def _check_device(*tensors: torch.Tensor) -> torch.device:
+    dev = tensors[0].device
+    if dev.type != "cuda":
+        raise RuntimeError(
+            "ragged_dot runs on a ROCm device only (tensors must be on 'cuda'); there is no CPU path. "
+            "interpret=True of the reference (the Pallas interpreter) has no counterpart here."
+        )
+    for t in tensors:
+        if t.device != dev:
+            raise RuntimeError("all operands must live on the same device")
+    return dev
+
+
+def _group_sizes_i32(group_sizes, dev: torch.device) -> torch.Tensor:
+    gs = torch.as_tensor(group_sizes)
+    if gs.dtype != torch.int32:
+        gs = gs.to(torch.int32)
+    return gs.to(dev).contiguous()
+
+
+def _stream_ptr(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _plan_ref(plan: Optional[_capi.Plan]):
+    return ctypes.byref(plan) if plan is not None else None
+
+
+def _gmm_fwd(x, A, group_sizes, block_m, block_k, block_n, trans_rhs, interpret, compute_dtype, acc_dtype, chunk_m,
+             plan: Optional[_capi.Plan] = None) -> torch.Tensor:
+    """gpu_ragged_dot.py:171-228 (_gpu_gmm_fwd): checks, planning, one call across the C ABI."""
+    if interpret:
+        raise NotImplementedError("interpret=True (Pallas interpreter) has no counterpart; kernels run on the GPU only")
+    assert A.ndim == 3 and x.ndim == 2, f"but {A.ndim=} {x.ndim=}"  # :188
+    gs_host_shape = tuple(torch.as_tensor(group_sizes).shape)
+    assert tuple(A.shape[:1]) == gs_host_shape, f"{A.shape[:1]=} != {gs_host_shape=}"  # :189
+    m, k = x.shape
+    g = A.shape[0]
+    n = A.shape[-1] if not trans_rhs else A.shape[-2]  # :190
+    k_rhs = A.shape[-2] if not trans_rhs else A.shape[-1]
+    assert k_rhs == k, f"contraction mismatch: x has k={k}, A has {k_rhs}"
+    assert chunk_m >= 1
+    planner.normalize_gmm_blocks(block_m, block_k, block_n, m, k, n)  # validates the request like :194-197
+    dev = _check_device(x, A)
+    code = _dtype_code(x, compute_dtype, acc_dtype)
+    if A.dtype != x.dtype:
+        raise TypeError(f"x is {x.dtype} but A is {A.dtype}")
+    x, A = x.contiguous(), A.contiguous()
+    gs = _group_sizes_i32(group_sizes, dev)
+    y = torch.empty((m, n), dtype=x.dtype, device=dev)  # :210
+    if plan is None:
+        plan = planner.select_plan(_capi.OP_GMM_TRANS if trans_rhs else _capi.OP_GMM, m, k, n, g, block_m, block_k, block_n)
+    ws_bytes = _capi.lib.rd_gmm_workspace_bytes(m, g, _plan_ref(plan))
+    ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _capi.check(
+            _capi.lib.rd_gmm(_stream_ptr(dev), x.data_ptr(), A.data_ptr(), gs.data_ptr(), y.data_ptr(), m, k, n, g,
+                             int(bool(trans_rhs)), code, _plan_ref(plan), ws.data_ptr(), ws.numel())
+        )
+    return y
+
+
+def _tgmm_fwd(x, y, group_sizes, block_m, block_k, block_n, interpret, compute_dtype, acc_dtype, chunk_m,
+              plan: Optional[_capi.Plan] = None) -> torch.Tensor:
+    """gpu_ragged_dot.py:287-342 (_gpu_tgmm_fwd)."""
+    del chunk_m  # :303
+    if interpret:
+        raise NotImplementedError("interpret=True (Pallas interpreter) has no counterpart; kernels run on the GPU only")
+    assert y.ndim == 2 and x.ndim == 2 and x.shape[0] == y.shape[0]  # :304
+    (m, k), n = x.shape, y.shape[-1]
+    gs_t = torch.as_tensor(group_sizes)
+    g = gs_t.numel()
+    planner.normalize_tgmm_blocks(block_m, block_k, block_n, m, k, n)  # :308-314
+    dev = _check_device(x, y)
+    code = _dtype_code(x, compute_dtype, acc_dtype)
+    if y.dtype != x.dtype:
+        raise TypeError(f"x is {x.dtype} but y is {y.dtype}")
+    x, y = x.contiguous(), y.contiguous()
+    gs = _group_sizes_i32(gs_t, dev)
+    out = torch.empty((g, k, n), dtype=x.dtype, device=dev)  # :324
+    if plan is None:
+        plan = planner.select_plan(_capi.OP_TGMM, m, k, n, g, block_m, block_k, block_n)
+    ws_bytes = _capi.lib.rd_tgmm_workspace_bytes(m, g, _plan_ref(plan))
+    ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _capi.check(
+            _capi.lib.rd_tgmm(_stream_ptr(dev), x.data_ptr(), y.data_ptr(), gs.data_ptr(), out.data_ptr(), m, k, n, g,
+                              code, _plan_ref(plan), ws.data_ptr(), ws.numel())
+        )
+    return out
+
+
+class _GmmFn(torch.autograd.Function):
+    """The custom VJP of gpu_ragged_dot.py:360-405, as a torch autograd node."""
+
+    @staticmethod
+    def forward(ctx, x, A, group_sizes, hp):
+        ctx.hp = hp
+        ctx.save_for_backward(x, A, group_sizes)  # residuals (x, A, group_sizes), :227
+        return _gmm_fwd(x, A, group_sizes, **hp)
+
+    @staticmethod
+    def backward(ctx, do):
+        x, A, group_sizes = ctx.saved_tensors
+        hp = dict(ctx.hp)
+        trans_rhs = hp.pop("trans_rhs")
+        hp.pop("plan", None)
+        do = do.contiguous()
+        dx = dA = None
+        if ctx.needs_input_grad[0]:
+            dx = _gmm_fwd(do, A, group_sizes, **hp, trans_rhs=not trans_rhs)  # :400
+        if ctx.needs_input_grad[1]:
+            thp = {k_: v for k_, v in hp.items()}
+            dA = _tgmm_fwd(x, do, group_sizes, **thp) if not trans_rhs else _tgmm_fwd(do, x, group_sizes, **thp)  # :401
+        return dx, dA, None, None  # group_sizes gets no cotangent, :402
+
+
+class _TgmmFn(torch.autograd.Function):
+    """tgmm with the VJP gpu_ragged_dot.py:431-450 intends: dx = gmm(y, do, trans_rhs=True), dy = gmm(x, do)."""
+
+    @staticmethod
+    def forward(ctx, x, y, group_sizes, hp):
+        ctx.hp = hp
+        ctx.save_for_backward(x, y, group_sizes)
+        return _tgmm_fwd(x, y, group_sizes, **hp)
+
+    @staticmethod
+    def backward(ctx, do):
+        x, y, group_sizes = ctx.saved_tensors
+        hp = dict(ctx.hp)
+        hp.pop("plan", None)
+        do = do.contiguous()
+        dx = dy = None
+        if ctx.needs_input_grad[0]:
+            dx = _gmm_fwd(y, do, group_sizes, **hp, trans_rhs=True)
+        if ctx.needs_input_grad[1]:
+            dy = _gmm_fwd(x, do, group_sizes, **hp, trans_rhs=False)
+        return dx, dy, None, None
+
+
+def gmm(
+    x: torch.Tensor,  # [m, k]
+    A: torch.Tensor,  # [g, k, n]  ([g, n, k] with trans_rhs)
+    group_sizes,  # [g]
+    block_m: int = DEFAULT_BLOCK_M,
+    block_k: int = DEFAULT_BLOCK_K,
+    block_n: int = DEFAULT_BLOCK_N,
+    trans_rhs: bool = False,
+    interpret: bool = False,
+    compute_dtype=None,
+    acc_dtype=torch.float32,
+    num_warps: Optional[int] = None,
+    num_stages: Optional[int] = None,
+    chunk_m: int = CHUNK_M,
+) -> torch.Tensor:
+    """Ragged dot corresponding to jax.lax.ragged_dot: (m, k) x (g, k, n) -> (m, n).  gpu_ragged_dot.py:362-380.
+
+    ``num_warps`` / ``num_stages`` are Triton knobs of the reference and are accepted and ignored; ``chunk_m`` is
+    validated only (the kernels split groups by their own tile height).
+    """
+    del num_warps, num_stages
+    hp = dict(block_m=block_m, block_k=block_k, block_n=block_n, trans_rhs=trans_rhs, interpret=interpret,
+              compute_dtype=compute_dtype, acc_dtype=acc_dtype, chunk_m=chunk_m)
+    if torch.is_grad_enabled() and (x.requires_grad or A.requires_grad):
+        gs = _group_sizes_i32(group_sizes, x.device)
+        return _GmmFn.apply(x, A, gs, hp)
+    return _gmm_fwd(x, A, group_sizes, **hp)
+
+
+def tgmm(
+    x: torch.Tensor,  # [m, k]
+    y: torch.Tensor,  # [m, n]
+    group_sizes,  # [g]
+    block_m: int = DEFAULT_BLOCK_M,
+    block_k: int = DEFAULT_BLOCK_K,
+    block_n: int = DEFAULT_BLOCK_N,
+    interpret: bool = False,
+    compute_dtype=None,
+    acc_dtype=torch.float32,
+    num_warps: Optional[int] = None,
+    num_stages: Optional[int] = None,
+    chunk_m: int = CHUNK_M,
+) -> torch.Tensor:
+    """Transposed ragged dot: (m, k) x (m, n) -> (g, k, n).  gpu_ragged_dot.py:411-428."""
+    del num_warps, num_stages
+    hp = dict(block_m=block_m, block_k=block_k, block_n=block_n, interpret=interpret, compute_dtype=compute_dtype,
+              acc_dtype=acc_dtype, chunk_m=chunk_m)
+    if torch.is_grad_enabled() and (x.requires_grad or y.requires_grad):
+        gs = _group_sizes_i32(group_sizes, x.device)
+        return _TgmmFn.apply(x, y, gs, hp)
+    return _tgmm_fwd(x, y, group_sizes, **hp)
+
+
+ragged_dot = gmm  # gpu_ragged_dot.py:406
+trans_ragged_dot = tgmm  # gpu_ragged_dot.py:454
+
+
+def ragged_dot_vjp(x, A, group_sizes, dout, trans_rhs: bool = False, **hp):
+    """Forward plus the VJP rule of gpu_ragged_dot.py:383-402 in one call: returns (y, dx, dA)."""
+    kw = dict(block_m=DEFAULT_BLOCK_M, block_k=DEFAULT_BLOCK_K, block_n=DEFAULT_BLOCK_N, interpret=False,
+              compute_dtype=None, acc_dtype=torch.float32, chunk_m=CHUNK_M)
+    kw.update(hp)
+    y = _gmm_fwd(x, A, group_sizes, **kw, trans_rhs=trans_rhs)
+    dx = _gmm_fwd(dout, A, group_sizes, **kw, trans_rhs=not trans_rhs)
+    dA = _tgmm_fwd(x, dout, group_sizes, **kw) if not trans_rhs else _tgmm_fwd(dout, x, group_sizes, **kw)
+    return y, dx, dA
+
+
+def make_group_metadata(group_sizes, m: int, chunk_m: int = CHUNK_M):
+    """The scheduling map of gpu_ragged_dot.py:70-90, computed on the device.
+
+    Returns (group_offsets[g], row_it2group[U], row_it2it_in_group[U], total_row_its[1]) as int32 device tensors.
+    """
+    gs_t = torch.as_tensor(group_sizes)
+    if gs_t.device.type != "cuda":
+        gs_t = gs_t.to("cuda")
+    dev = gs_t.device
+    gs = _group_sizes_i32(gs_t, dev)
+    g = gs.numel()
+    U = _capi.lib.rd_sched_map_len(m, g, chunk_m)
+    if U < 0:
+        _capi.check(U)
+    offs = torch.empty(g, dtype=torch.int32, device=dev)
+    t2g = torch.empty(U, dtype=torch.int32, device=dev)
+    t2it = torch.empty(U, dtype=torch.int32, device=dev)
+    total = torch.empty(1, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _capi.check(
+            _capi.lib.rd_sched_map(_stream_ptr(dev), gs.data_ptr(), g, m, chunk_m, offs.data_ptr(), t2g.data_ptr(),
+                                   t2it.data_ptr(), total.data_ptr())
+        )
+    return offs, t2g, t2it, total

@@ -1,0 +1,99 @@
+/* C ABI of the MI355X (gfx950) ragged_dot kernels.
+ *
+ * This is the boundary the reference crosses at its two pl.pallas_call sites
+ * (gpu_ragged_dot.py:217-226 for gmm, :331-340 for tgmm): device buffers in, device buffers out, everything
+ * enqueued on the caller's stream, no host synchronisation.  Plain C types only.
+ *
+ * Conventions
+ *  - every pointer is a device pointer unless it says "host"; the caller owns all buffers, including the
+ *    workspace; the library never allocates or frees device memory and never synchronises;
+ *  - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *  - matrices are dense row-major; element type is selected by `dtype` (RD_DTYPE_*), output type = input type
+ *    (gpu_ragged_dot.py:210,324), accumulation is always fp32 (acc_dtype, gpu_ragged_dot.py:119,251);
+ *  - return value 0 = success; negative = RD_ERR_*; the text of the last error of the calling thread is
+ *    available from rd_last_error().  Nothing here aborts the process;
+ *  - no host reads of device data: the launch grid is the static bound ceil(m / tile_m) + g of
+ *    gpu_ragged_dot.py:212, so every entry point can be recorded into a HIP graph.
+ */
+#ifndef RAGGED_DOT_HIP_H_
+#define RAGGED_DOT_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RD_ABI_VERSION 1
+
+enum rd_dtype { RD_DTYPE_BF16 = 0, RD_DTYPE_F32 = 1 };
+
+enum rd_status {
+  RD_OK = 0,
+  RD_ERR_INVALID_ARGUMENT = -1, /* bad shape / null pointer / unknown enum */
+  RD_ERR_UNSUPPORTED = -2,      /* valid request that this build has no kernel for */
+  RD_ERR_WORKSPACE = -3,        /* workspace too small or misaligned */
+  RD_ERR_HIP = -4               /* a HIP runtime call failed; see rd_last_error() */
+};
+
+/* One compiled tile shape.  `id` indexes the table rd_num_variants()/rd_get_variant() expose. */
+typedef struct rd_variant_info {
+  int id;
+  int tile_m, tile_n, tile_k; /* macro-tile: rows x columns x contraction slab */
+  int waves_m, waves_n;       /* wavefront grid inside a work-group (64 lanes each) */
+  int vec;                    /* 1: needs 16-byte row pitches (k % 8 == 0 and n % 8 == 0 for bf16) */
+  char name[48];
+} rd_variant_info;
+
+/* Launch plan for one call; the host planner (or the caller) fills it.  Zero-initialised = library defaults. */
+typedef struct rd_plan {
+  int variant; /* index into the variant table, or -1: let the library choose by shape */
+  int group_m; /* row tiles per band of the tile walk (L2 reuse); 0 = default */
+  int decode_nb; /* rd_gmm only: > 0 selects the skinny-m streaming kernel with this many columns per work-group */
+} rd_plan;
+
+int rd_abi_version(void);
+const char* rd_last_error(void); /* host pointer, valid until the thread's next failing call */
+
+int rd_num_variants(void);
+int rd_get_variant(int id, rd_variant_info* out /* host */);
+
+/* The library's own shape-based choice (what variant = -1 resolves to); op: 0 gmm, 1 gmm trans_rhs, 2 tgmm. */
+int rd_default_plan(int op, int m, int k, int n, int g, int dtype, rd_plan* out /* host */);
+
+/* ---- scheduling map --------------------------------------------------------------------------------------
+ * Replaces _make_gmm_group_metadata (gpu_ragged_dot.py:70-90).  Bit-exact int32 outputs:
+ *   group_offsets[g]                = exclusive prefix sum of group_sizes                         (:86)
+ *   row_it2group[U], row_it2it_in_group[U],  U = ceil(m / chunk_m) + g                            (:77-82)
+ *   total_row_its[1]                = sum(ceil(group_sizes / chunk_m))                            (:89)
+ * Requires g >= 1, m >= 0, chunk_m >= 1. */
+int rd_sched_map(void* stream, const int32_t* group_sizes, int g, int m, int chunk_m, int32_t* group_offsets,
+                 int32_t* row_it2group, int32_t* row_it2it_in_group, int32_t* total_row_its);
+
+/* Number of entries U of the two per-tile arrays (gpu_ragged_dot.py:77, :212). */
+int rd_sched_map_len(int m, int g, int chunk_m);
+
+/* ---- gmm: y[m, n] = ragged x[m, k] . A ----------------------------------------------------------------------
+ * Replaces the "gpu_gmm" pallas_call (gpu_ragged_dot.py:93-165, 217-226).
+ *   A is [g, k, n] (trans_rhs = 0) or [g, n, k] (trans_rhs = 1, gpu_ragged_dot.py:139-144, :190).
+ *   Rows of group i are [offset_i, offset_i + group_sizes[i]); rows >= sum(group_sizes) of y are set to zero
+ *   (:155-165) -- also when every group is empty.  Groups that would run past m are clipped to m.
+ * Workspace: rd_gmm_workspace_bytes() bytes, 256-byte aligned; holds the scheduling map. */
+size_t rd_gmm_workspace_bytes(int m, int g, const rd_plan* plan /* host, may be NULL */);
+int rd_gmm(void* stream, const void* x, const void* A, const int32_t* group_sizes, void* y, int m, int k, int n,
+           int g, int trans_rhs, int dtype, const rd_plan* plan /* host, may be NULL */, void* workspace,
+           size_t workspace_bytes);
+
+/* ---- tgmm: dA[g, k, n] = x[rows of g, :]^T . dy[rows of g, :] -----------------------------------------------
+ * Replaces the "gpu_tgmm" pallas_call (gpu_ragged_dot.py:231-281, 331-340).  Slices of empty groups are zero
+ * (:277-281).  x is [m, k], dy is [m, n]. */
+size_t rd_tgmm_workspace_bytes(int m, int g, const rd_plan* plan /* host, may be NULL */);
+int rd_tgmm(void* stream, const void* x, const void* dy, const int32_t* group_sizes, void* dA, int m, int k,
+            int n, int g, int dtype, const rd_plan* plan /* host, may be NULL */, void* workspace,
+            size_t workspace_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RAGGED_DOT_HIP_H_ */

@@ -1,0 +1,317 @@
+"""CPU oracle for the ragged_dot hot path.  TEST INFRASTRUCTURE ONLY.
+
+This module is a numpy restatement of the algorithm in the reference's
+``gpu_ragged_dot.py``.  It exists to *check* the HIP kernels; nothing in the
+shipped package may import it.  Only ``tests/``, ``__graft_entry__.smoke()``
+and the ``cpu_baseline`` leg of ``bench.py`` use it.
+
+Every function names the reference lines it restates.  How each one is pinned
+(``tests/test_oracle.py``):
+
+* ``make_gmm_group_metadata``  - hand-computed known answers, the closed form
+  ``repeat(arange(g), bpg)`` / ``concat(arange(b))``, and interval invariants.
+* ``gmm`` / ``tgmm`` (definition) - special cases that reduce to library
+  routines written independently of this file (g=1 -> ``numpy.matmul``; equal
+  groups -> ``numpy.einsum`` batched matmul; all-ones inputs -> every valid
+  output equals the contraction length, the reference's own
+  ``random_inputs=False`` case, tests.py:67,103); trans_rhs on ``A.mT`` equals
+  the plain product (tests.py:156-161).
+* ``gmm_blocked`` / ``tgmm_blocked`` (the reference's work-item / row-block /
+  K-block loop nest) - against the definition above on the reference's own
+  test grid (tests.py:91-105), incl. the non-multiples 171/58/77.
+* ``gmm_vjp`` - adjoint identities <dout, gmm(x,A)> = <dlhs, x> = <drhs, A> in
+  float64, which fix the wiring of gpu_ragged_dot.py:400-401 with no outside
+  oracle, plus central finite differences.
+* block-size rules - table tests of the integer rules.
+
+The reference holds no golden vectors or fixtures on disk (tests.py compares
+live against jax.lax.ragged_dot_general on a GPU), and JAX is not installed
+here, so exact agreement with XLA's own rounding/accumulation order is
+"parity unpinned"; everything arithmetic is pinned as listed.
+"""
+
+from __future__ import annotations
+
+from typing import NamedTuple
+
+import numpy as np
+
+DEFAULT_BLOCK_M = 64  # gpu_ragged_dot.py:34
+DEFAULT_BLOCK_N = 64  # gpu_ragged_dot.py:35
+DEFAULT_BLOCK_K = 64  # gpu_ragged_dot.py:36
+CHUNK_M = 512  # gpu_ragged_dot.py:42
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# bfloat16 on the host (numpy has no bf16): round-to-nearest-even through the bit pattern
+# ---------------------------------------------------------------------------------------------------------------------
+
+
+def f32_to_bf16_bits(a: np.ndarray) -> np.ndarray:
+    """float32 -> bf16 bit pattern (uint16), round to nearest even, NaN kept quiet."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+    bias = ((u >> np.uint32(16)) & np.uint32(1)) + np.uint32(0x7FFF)
+    r = ((u + bias) >> np.uint32(16)).astype(np.uint16)
+    nan = (u & np.uint32(0x7FFFFFFF)) > np.uint32(0x7F800000)
+    r = np.where(nan, ((u >> np.uint32(16)) | np.uint32(0x0040)).astype(np.uint16), r)
+    return r
+
+
+def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(b, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def round_to(a: np.ndarray, dtype: str) -> np.ndarray:
+    """Round a float array to ``dtype`` ('bfloat16' | 'float32') and return it as float32 values."""
+    if dtype == "bfloat16":
+        return bf16_bits_to_f32(f32_to_bf16_bits(a)).reshape(np.shape(a))
+    if dtype == "float32":
+        return np.asarray(a, dtype=np.float32)
+    raise ValueError(f"unsupported dtype {dtype!r}")
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# scheduling map  (gpu_ragged_dot.py:60-90)
+# ---------------------------------------------------------------------------------------------------------------------
+
+
+class GMMGroupLookupMetadata(NamedTuple):  # gpu_ragged_dot.py:60-67
+    group_sizes: np.ndarray
+    group_offsets: np.ndarray
+    row_it2group: np.ndarray
+    row_it2it_in_group: np.ndarray
+    total_row_its: np.ndarray
+
+
+def make_gmm_group_metadata(group_sizes: np.ndarray, m: int, chunk_m: int) -> GMMGroupLookupMetadata:
+    """gpu_ragged_dot.py:70-90, the 2-D shifted-iota mask construction, in int32 throughout."""
+    gs = np.asarray(group_sizes, dtype=np.int32)
+    g = gs.size
+    c = np.int32(chunk_m)
+    bpg = (gs + c - np.int32(1)) // c  # :73
+    boff = (np.cumsum(bpg, dtype=np.int32) - bpg).astype(np.int32)  # :76
+    ub = (m + chunk_m - 1) // chunk_m + g  # :77
+    iota = np.arange(ub, dtype=np.int32)[None, :] - boff[:, None]  # :78
+    mask = (iota >= 0) & (iota < bpg[:, None])  # :79
+    row_it2group = np.sum(np.where(mask, np.arange(g, dtype=np.int32)[:, None], 0), 0, dtype=np.int32)  # :81
+    row_it2it = np.sum(np.where(mask, iota, 0), 0, dtype=np.int32)  # :82
+    return GMMGroupLookupMetadata(
+        group_sizes=gs,
+        group_offsets=(np.cumsum(gs, dtype=np.int32) - gs).astype(np.int32),  # :86
+        row_it2group=row_it2group.reshape(ub).astype(np.int32),
+        row_it2it_in_group=row_it2it.reshape(ub).astype(np.int32),
+        total_row_its=np.asarray(np.sum(bpg, dtype=np.int32), dtype=np.int32),  # :89
+    )
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# host planning rules
+# ---------------------------------------------------------------------------------------------------------------------
+
+
+def next_power_of_2(x: int) -> int:
+    """pl.next_power_of_2: smallest power of two >= x (x >= 0; 0 -> 1)."""
+    if x < 0:
+        raise ValueError("next_power_of_2 needs x >= 0")
+    return 1 if x == 0 else 1 << (int(x) - 1).bit_length()
+
+
+def gmm_block_sizes(block_m: int, block_k: int, block_n: int, m: int, k: int, n: int) -> tuple[int, int, int]:
+    """gpu_ragged_dot.py:194-197: next_pow2(min(b, size)); only block_k and block_n are raised to 16."""
+    bm, bk, bn = [next_power_of_2(min(b, s)) for b, s in zip([block_m, block_k, block_n], [m, k, n])]
+    return bm, max(bk, 16), max(bn, 16)
+
+
+def tgmm_block_sizes(block_m: int, block_k: int, block_n: int, m: int, k: int, n: int) -> tuple[int, int, int]:
+    """gpu_ragged_dot.py:308-314: all three are raised to 16 (the 4th zip entry is dropped by zip)."""
+    block_m, block_n = min(block_m, m), min(block_n, n)
+    bm, bk, bn = [max(next_power_of_2(min(b, s)), 16) for b, s in zip([block_m, block_k, block_n], [m, k, n])]
+    return bm, bk, bn
+
+
+def gmm_grid(m: int, n: int, g: int, block_n: int, chunk_m: int) -> tuple[int, int]:
+    """gpu_ragged_dot.py:212-213."""
+    return ((m + chunk_m - 1) // chunk_m + g, -(-n // block_n))
+
+
+def tgmm_grid(k: int, n: int, g: int, block_k: int, block_n: int) -> tuple[int, int, int]:
+    """gpu_ragged_dot.py:326."""
+    return (g, -(-k // block_k), -(-n // block_n))
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# definition: block-diagonal products (what jax.lax.ragged_dot_general computes for the two dimension-number
+# sets of tests.py:31-36), in float32 on the stored values, rounded once to the output dtype
+# ---------------------------------------------------------------------------------------------------------------------
+
+
+def _offsets(group_sizes: np.ndarray) -> np.ndarray:
+    gs = np.asarray(group_sizes, dtype=np.int64)
+    return np.concatenate([[0], np.cumsum(gs)])
+
+
+def gmm(x, A, group_sizes, trans_rhs: bool = False, out_dtype: str = "bfloat16", acc=np.float32) -> np.ndarray:
+    """y[rows of group g] = x[rows] @ A[g] (or @ A[g].T), rows >= sum(group_sizes) are zero.
+
+    gpu_ragged_dot.py:108-150 (which rows a work item owns; dtype flow :116-119,145-149) and :155-165 (tail zero).
+    """
+    x = np.asarray(x, dtype=acc)
+    A = np.asarray(A, dtype=acc)
+    m = x.shape[0]
+    n = A.shape[-2] if trans_rhs else A.shape[-1]  # :190
+    off = _offsets(group_sizes)
+    y = np.zeros((m, n), dtype=acc)
+    for gi in range(A.shape[0]):
+        lo, hi = min(int(off[gi]), m), min(int(off[gi + 1]), m)
+        if hi > lo:
+            y[lo:hi] = x[lo:hi] @ (A[gi].T if trans_rhs else A[gi])
+    return round_to(y, out_dtype) if acc == np.float32 else y
+
+
+def tgmm(x, y, group_sizes, out_dtype: str = "bfloat16", acc=np.float32) -> np.ndarray:
+    """A_bar[g] = x[rows of g].T @ y[rows of g]; empty group -> zeros (gpu_ragged_dot.py:250-281)."""
+    x = np.asarray(x, dtype=acc)
+    y = np.asarray(y, dtype=acc)
+    m = x.shape[0]
+    off = _offsets(group_sizes)
+    g = len(off) - 1
+    out = np.zeros((g, x.shape[1], y.shape[1]), dtype=acc)
+    for gi in range(g):
+        lo, hi = min(int(off[gi]), m), min(int(off[gi + 1]), m)
+        if hi > lo:
+            out[gi] = x[lo:hi].T @ y[lo:hi]
+    return round_to(out, out_dtype) if acc == np.float32 else out
+
+
+def gmm_vjp(x, A, group_sizes, dout, trans_rhs: bool = False, out_dtype: str = "bfloat16", acc=np.float32):
+    """gpu_ragged_dot.py:383-402: dx = gmm(do, A, !trans_rhs); dA = tgmm(x, do) or tgmm(do, x); None for sizes."""
+    dx = gmm(dout, A, group_sizes, trans_rhs=not trans_rhs, out_dtype=out_dtype, acc=acc)  # :400
+    if not trans_rhs:
+        dA = tgmm(x, dout, group_sizes, out_dtype=out_dtype, acc=acc)  # :401
+    else:
+        dA = tgmm(dout, x, group_sizes, out_dtype=out_dtype, acc=acc)
+    return dx, dA, None
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# restatement of the reference's kernels as loop nests (small cases only: pure Python loops over programs)
+# ---------------------------------------------------------------------------------------------------------------------
+
+
+def gmm_blocked(
+    x,
+    A,
+    group_sizes,
+    block_m: int = DEFAULT_BLOCK_M,
+    block_k: int = DEFAULT_BLOCK_K,
+    block_n: int = DEFAULT_BLOCK_N,
+    trans_rhs: bool = False,
+    chunk_m: int = CHUNK_M,
+    out_dtype: str = "bfloat16",
+    fill: float = np.nan,
+) -> np.ndarray:
+    """The program grid of _gpu_gmm_fwd/_gpu_gmm_kernel, one Python iteration per program.
+
+    ``fill`` stands for the uninitialised output buffer the reference starts from: entries no program writes keep
+    it, so a test can see exactly which elements the reference defines (gpu_ragged_dot.py:150,155-165).
+    """
+    x = np.asarray(x, dtype=np.float32)
+    A = np.asarray(A, dtype=np.float32)
+    gs = np.asarray(group_sizes, dtype=np.int32)
+    m, k = x.shape
+    g = A.shape[0]
+    n = A.shape[-2] if trans_rhs else A.shape[-1]
+    bm, bk, bn = gmm_block_sizes(block_m, block_k, block_n, m, k, n)
+    md = make_gmm_group_metadata(gs, m, chunk_m)
+    grid = gmm_grid(m, n, g, bn, chunk_m)
+    y = np.full((m, n), fill, dtype=np.float32)
+    total = int(md.total_row_its)
+    last_offset = int(md.group_offsets[g - 1]) + int(gs[g - 1])  # :156
+    for i in range(grid[0]):
+        gi = int(md.row_it2group[i])  # :108-110
+        local_inc = chunk_m * int(md.row_it2it_in_group[i])  # :112
+        valid = i < total  # :113
+        group_sz = int(np.clip(int(gs[gi]) - local_inc, 0, chunk_m)) if valid else 0  # :114
+        for j in range(grid[1]):
+            c0, c1 = j * bn, min((j + 1) * bn, n)
+            if group_sz > 0:  # :121
+                start = int(md.group_offsets[gi]) + local_inc  # :124
+                for r in range(-(-group_sz // bm)):  # :153
+                    r0 = start + r * bm
+                    r1 = start + min((r + 1) * bm, group_sz)  # row mask :128
+                    acc = np.zeros((r1 - r0, c1 - c0), dtype=np.float32)  # :147
+                    for kk in range(-(-k // bk)):  # :148
+                        k0, k1 = kk * bk, min((kk + 1) * bk, k)  # inner mask :135
+                        xa = x[r0:r1, k0:k1]
+                        Ab = A[gi, c0:c1, k0:k1].T if trans_rhs else A[gi, k0:k1, c0:c1]  # :139-144
+                        acc = acc + (xa @ Ab).astype(np.float32)  # :145
+                    y[r0:r1, c0:c1] = round_to(acc, out_dtype)  # :149-150
+            if i == total - 1 and last_offset < m:  # :157
+                y[last_offset:m, c0:c1] = 0.0  # :160-165
+    return y
+
+
+def tgmm_blocked(
+    x,
+    y,
+    group_sizes,
+    block_m: int = DEFAULT_BLOCK_M,
+    block_k: int = DEFAULT_BLOCK_K,
+    block_n: int = DEFAULT_BLOCK_N,
+    out_dtype: str = "bfloat16",
+) -> np.ndarray:
+    """The program grid of _gpu_tgmm_fwd/_gpu_tgmm_kernel (gpu_ragged_dot.py:231-342)."""
+    x = np.asarray(x, dtype=np.float32)
+    y = np.asarray(y, dtype=np.float32)
+    gs = np.asarray(group_sizes, dtype=np.int32)
+    (m, k), n = x.shape, y.shape[-1]
+    g = gs.size
+    bm, bk, bn = tgmm_block_sizes(block_m, block_k, block_n, m, k, n)
+    group_offsets = (np.cumsum(gs, dtype=np.int32) - gs).astype(np.int32)  # :316
+    grid = tgmm_grid(k, n, g, bk, bn)
+    out = np.full((g, k, n), np.nan, dtype=np.float32)
+    for gi in range(grid[0]):
+        group_sz = int(gs[gi])  # :247
+        start = 0 if gi == 0 else int(group_offsets[gi])  # :256
+        for r in range(grid[1]):
+            k0, k1 = r * bk, min((r + 1) * bk, k)  # :259
+            for c in range(grid[2]):
+                c0, c1 = c * bn, min((c + 1) * bn, n)  # :261
+                if group_sz > 0:  # :253
+                    acc = np.zeros((k1 - k0, c1 - c0), dtype=np.float32)  # :272
+                    for ro in range(-(-group_sz // bm)):  # :273
+                        r0 = start + ro * bm
+                        r1 = start + min((ro + 1) * bm, group_sz)  # :265
+                        acc = acc + (x[r0:r1, k0:k1].T @ y[r0:r1, c0:c1]).astype(np.float32)  # :270
+                    out[gi, k0:k1, c0:c1] = round_to(acc, out_dtype)  # :274-275
+                else:  # :277-281
+                    out[gi, k0:k1, c0:c1] = 0.0
+    return out
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# the reference's test metric and group-size generator (tests.py)
+# ---------------------------------------------------------------------------------------------------------------------
+
+
+def err_fn(a, b, axis=-1, mask=None) -> np.ndarray:
+    """tests.py:74-79: relative L2 error along ``axis``; entries where mask is False count as 0."""
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    ax = axis if isinstance(axis, tuple) else (axis,)
+    err = np.sqrt(np.sum((a - b) ** 2, axis=ax)) / np.maximum(np.sqrt(np.sum(b**2, axis=ax)), 1e-7)
+    if mask is not None:
+        mask = np.asarray(mask).reshape(np.shape(mask) + (1,) * (err.ndim - np.ndim(mask)))
+        return np.where(mask, err, 0.0)
+    return err
+
+
+def generate_group_sizes(seed: int, g: int, target_m: int) -> np.ndarray:
+    """tests.py:51-57 with an explicit integer seed: round(target_m * softmax(N(0,1))), arg-max absorbs the residue."""
+    z = np.random.default_rng(seed).normal(size=(g,))
+    e = np.exp(z - np.max(z))
+    group_sizes = np.round(target_m * (e / np.sum(e))).astype(np.int32)
+    while np.sum(group_sizes) != target_m:
+        idx = np.argmax(group_sizes)
+        group_sizes[idx] = max(group_sizes[idx] + (target_m - np.sum(group_sizes)), 0)
+    return group_sizes

@@ -1,0 +1,257 @@
+"""GPU parity: the HIP kernels, called through the C ABI, against the numpy oracle on the same seeded inputs.
+
+Bars: scheduling map bit-exact; products within the reference's own per-row relative-L2 eps (tests.py:127,144,168,
+183) and within max|diff| <= 1e-2 * max|ref|; tail rows and empty groups exactly zero.
+"""
+
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import gpu_ragged_dot_amd as rd
+from gpu_ragged_dot_amd import _capi, workloads
+from oracle import ragged_dot_oracle as oracle
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# scheduling map: bit-exact
+# ---------------------------------------------------------------------------------------------------------------------
+
+def _map_cases():
+    cases = []
+    for name in ("tiny", "mixtral_fwd", "deepseek_fwd_bwd", "decode"):
+        w = workloads.WORKLOADS[name]
+        for chunk in (512, 256, 128, 64, 32, 8):
+            cases.append((f"{name}-c{chunk}", workloads.group_sizes(name), w.m, chunk))
+    rng = np.random.default_rng(7)
+    for i in range(12):
+        g = int(rng.integers(1, 40))
+        m = int(rng.integers(1, 3000))
+        fill = float(rng.choice([1.0, 0.7, 0.5, 0.0]))
+        gs = oracle.generate_group_sizes(i, g, int(round(m * fill)))
+        gs[rng.random(g) < 0.3] = 0
+        cases.append((f"rand{i}", gs, m, int(rng.choice([1, 8, 64, 512]))))
+    gs = rng.integers(0, 50, size=3000).astype(np.int32)  # more groups than one work-group scans at once
+    cases.append(("g3000", gs, int(gs.sum()) + 17, 16))
+    cases.append(("one-group", np.array([1000], np.int32), 1000, 8))
+    cases.append(("all-empty", np.zeros(5, np.int32), 64, 8))
+    cases.append(("m0", np.zeros(3, np.int32), 0, 8))
+    return cases
+
+
+@pytest.mark.parametrize("name,gs,m,chunk", _map_cases(), ids=[c[0] for c in _map_cases()])
+def test_sched_map_bit_exact(name, gs, m, chunk):
+    print(f"sched_map case={name} g={gs.size} m={m} chunk={chunk}", flush=True)
+    offs, t2g, t2it, total = rd.make_group_metadata(torch.from_numpy(gs), m, chunk)
+    ref = oracle.make_gmm_group_metadata(gs, m, chunk)
+    np.testing.assert_array_equal(offs.cpu().numpy(), ref.group_offsets)
+    np.testing.assert_array_equal(t2g.cpu().numpy(), ref.row_it2group)
+    np.testing.assert_array_equal(t2it.cpu().numpy(), ref.row_it2it_in_group)
+    assert int(total.item()) == int(ref.total_row_its)
+    assert t2g.dtype == torch.int32 and t2it.dtype == torch.int32 and offs.dtype == torch.int32
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# the reference's test grid (tests.py:91-184), bf16
+# ---------------------------------------------------------------------------------------------------------------------
+
+GRID = util.reference_grid(40)
+
+
+@pytest.mark.parametrize("c", GRID, ids=[util.case_id(c) for c in GRID])
+def test_ragged_dot_grid(c):
+    """tests.py:119-128 plus: the tail is exactly zero."""
+    print("gmm fwd", c, flush=True)
+    lhs, rhs, _, gs, target_m = util.make_case(c["seed"], c["m"], c["k"], c["n"], c["g"], c["fill_in"], c["random_inputs"])
+    y = rd.gmm(util.bf16_dev(lhs), util.bf16_dev(rhs), torch.from_numpy(gs), block_m=c["block_m"], block_k=c["block_k"],
+               block_n=c["block_n"], chunk_m=c["chunk_m"])
+    y = util.to_np(y)
+    y_ref = oracle.gmm(lhs, rhs, gs)
+    util.assert_close_rows(y, y_ref, target_m, util.BF16_EPS, "y")
+    assert not np.any(y[target_m:]), "rows past sum(group_sizes) must be exactly zero"
+    if not c["random_inputs"]:
+        assert np.all(y[:target_m] == c["k"])  # all-ones inputs: every valid output is exactly k
+
+
+@pytest.mark.parametrize("trans_rhs", [False, True], ids=["A", "At"])
+@pytest.mark.parametrize("c", GRID[:24], ids=[util.case_id(c) for c in GRID[:24]])
+def test_ragged_dot_diff_grid(c, trans_rhs):
+    """tests.py:130-171: forward and both cotangents through autograd, with A given as [g,k,n] or [g,n,k]."""
+    print("gmm vjp", c, "trans_rhs", trans_rhs, flush=True)
+    lhs, rhs, dout, gs, target_m = util.make_case(c["seed"], c["m"], c["k"], c["n"], c["g"], c["fill_in"], c["random_inputs"])
+    rhs_in = np.ascontiguousarray(np.swapaxes(rhs, 1, 2)) if trans_rhs else rhs
+    x_t = util.bf16_dev(lhs).requires_grad_(True)
+    A_t = util.bf16_dev(rhs_in).requires_grad_(True)
+    o = rd.gmm(x_t, A_t, torch.from_numpy(gs), block_m=c["block_m"], block_k=c["block_k"], block_n=c["block_n"],
+               chunk_m=c["chunk_m"], trans_rhs=trans_rhs)
+    dlhs, drhs = torch.autograd.grad(o, (x_t, A_t), util.bf16_dev(dout))
+    o_ref = oracle.gmm(lhs, rhs_in, gs, trans_rhs=trans_rhs)
+    dlhs_ref, drhs_ref, _ = oracle.gmm_vjp(lhs, rhs_in, gs, dout, trans_rhs=trans_rhs)
+    util.assert_close_rows(util.to_np(o), o_ref, target_m, util.BF16_EPS, "o")
+    util.assert_close_rows(util.to_np(dlhs), dlhs_ref, target_m, util.BF16_EPS, "dlhs")
+    drhs = util.to_np(drhs)
+    util.assert_close_groups(drhs, drhs_ref, gs != 0, util.BF16_EPS, "drhs")
+    assert not np.any(drhs[gs == 0]), "cotangent of an empty group's weights must be exactly zero"
+    assert not np.any(util.to_np(dlhs)[target_m:])
+
+
+@pytest.mark.parametrize("c", GRID[:24], ids=[util.case_id(c) for c in GRID[:24]])
+def test_trans_ragged_dot_grid(c):
+    """tests.py:173-184."""
+    print("tgmm", c, flush=True)
+    lhs, _, dout, gs, _ = util.make_case(c["seed"], c["m"], c["k"], c["n"], c["g"], c["fill_in"], c["random_inputs"])
+    out = rd.tgmm(util.bf16_dev(lhs), util.bf16_dev(dout), torch.from_numpy(gs), block_m=c["block_m"],
+                  block_k=c["block_k"], block_n=c["block_n"], chunk_m=c["chunk_m"])
+    out = util.to_np(out)
+    ref = oracle.tgmm(lhs, dout, gs)
+    util.assert_close_groups(out, ref, gs != 0, util.TGMM_BF16_EPS, "tgmm")
+    assert not np.any(out[gs == 0])
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# every compiled tile shape, all three operand layouts
+# ---------------------------------------------------------------------------------------------------------------------
+
+def _variant_ids():
+    return [(v.id, v.name.decode(), v.vec) for v in _capi.variants()]
+
+
+@pytest.mark.parametrize("vid,vname,vec", _variant_ids(), ids=[v[1] for v in _variant_ids()])
+@pytest.mark.parametrize("shape", [(700, 328, 520, 5), (300, 64, 264, 3)], ids=["m700k328n520g5", "m300k64n264g3"])
+def test_every_variant(vid, vname, vec, shape):
+    m, k, n, g = shape
+    print(f"variant {vname} shape {shape}", flush=True)
+    lhs, rhs, dout, gs, target_m = util.make_case(3, m, k, n, g, 0.9, True, scale_rhs=True)
+    gs[1] = 0 if g > 2 else gs[1]
+    target_m = int(gs.sum())
+    plan = _capi.Plan(vid, 3, 0)
+    gs_t = torch.from_numpy(gs)
+    hp = dict(block_m=64, block_k=64, block_n=64, interpret=False, compute_dtype=None, acc_dtype=torch.float32, chunk_m=512)
+    from gpu_ragged_dot_amd import ops
+    y = ops._gmm_fwd(util.bf16_dev(lhs), util.bf16_dev(rhs), gs_t, **hp, trans_rhs=False, plan=plan)
+    yt = ops._gmm_fwd(util.bf16_dev(lhs), util.bf16_dev(np.ascontiguousarray(np.swapaxes(rhs, 1, 2))), gs_t, **hp,
+                      trans_rhs=True, plan=plan)
+    dA = ops._tgmm_fwd(util.bf16_dev(lhs), util.bf16_dev(dout), gs_t, **hp, plan=plan)
+    y_ref = oracle.gmm(lhs, rhs, gs)
+    util.assert_close_rows(util.to_np(y), y_ref, target_m, util.BF16_EPS, "y")
+    util.assert_close_rows(util.to_np(yt), y_ref, target_m, util.BF16_EPS, "y (trans_rhs)")
+    assert not np.any(util.to_np(y)[target_m:]) and not np.any(util.to_np(yt)[target_m:])
+    dA_ref = oracle.tgmm(lhs, dout, gs)
+    util.assert_close_groups(util.to_np(dA), dA_ref, gs != 0, util.TGMM_BF16_EPS, "dA")
+    assert not np.any(util.to_np(dA)[gs == 0])
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# configuration C1 (tiny) with its exact recipe, and the other configurations' shapes
+# ---------------------------------------------------------------------------------------------------------------------
+
+def test_tiny_config_fwd_vjp():
+    print("tiny config", flush=True)
+    x, A, dout, gs = workloads.make_inputs("tiny")
+    assert gs.cpu().tolist() == [116, 133, 132, 131]
+    y, dx, dA = rd.ragged_dot_vjp(x, A, gs, dout)
+    xn, An, dn, gsn = util.to_np(x), util.to_np(A), util.to_np(dout), gs.cpu().numpy()
+    dx_ref, dA_ref, _ = oracle.gmm_vjp(xn, An, gsn, dn)
+    util.assert_close_rows(util.to_np(y), oracle.gmm(xn, An, gsn), 512, util.BF16_EPS, "y")
+    util.assert_close_rows(util.to_np(dx), dx_ref, 512, util.BF16_EPS, "dlhs")
+    util.assert_close_groups(util.to_np(dA), dA_ref, gsn != 0, util.TGMM_BF16_EPS, "drhs")
+
+
+def test_decode_config():
+    print("decode config", flush=True)
+    x, A, _, gs = workloads.make_inputs("decode")
+    gsn = gs.cpu().numpy()
+    assert int(gsn.sum()) == 64 and int((gsn > 0).sum()) == 53
+    y_ref = oracle.gmm(util.to_np(x), util.to_np(A), gsn)
+    for nb in (32, 64, 128):
+        from gpu_ragged_dot_amd import ops
+        y = ops._gmm_fwd(x, A, gs, 64, 64, 64, False, False, None, torch.float32, 512, plan=_capi.Plan(-1, 0, nb))
+        util.assert_close_rows(util.to_np(y), y_ref, 64, util.BF16_EPS, f"decode nb={nb}")
+    y = rd.ragged_dot(x, A, gs)  # default plan for this shape is the streaming kernel
+    util.assert_close_rows(util.to_np(y), y_ref, 64, util.BF16_EPS, "decode default")
+
+
+def test_decode_kernel_long_groups_and_tail():
+    """More rows per group than the streaming kernel holds at once, a zero tail, and a ragged last column block."""
+    print("decode long groups", flush=True)
+    m, k, n, g = 40, 520, 200, 6
+    lhs, rhs, _, _, _ = util.make_case(5, m, k, n, g, 1.0, True, scale_rhs=True)
+    gs = np.array([0, 11, 1, 0, 9, 5], np.int32)  # sum 26 < 40
+    from gpu_ragged_dot_amd import ops
+    for nb in (32, 64, 128):
+        y = ops._gmm_fwd(util.bf16_dev(lhs), util.bf16_dev(rhs), torch.from_numpy(gs), 64, 64, 64, False, False, None,
+                         torch.float32, 512, plan=_capi.Plan(-1, 0, nb))
+        y = util.to_np(y)
+        util.assert_close_rows(y, oracle.gmm(lhs, rhs, gs), 26, util.BF16_EPS, f"nb={nb}")
+        assert not np.any(y[26:])
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# what the reference leaves undefined or never checks
+# ---------------------------------------------------------------------------------------------------------------------
+
+def _raw_gmm(x, A, gs, y, trans_rhs=False, plan=None):
+    m, k = x.shape
+    g = A.shape[0]
+    n = A.shape[1] if trans_rhs else A.shape[2]
+    ws = torch.empty(_capi.lib.rd_gmm_workspace_bytes(m, g, None), dtype=torch.uint8, device="cuda")
+    rc = _capi.lib.rd_gmm(torch.cuda.current_stream().cuda_stream, x.data_ptr(), A.data_ptr(), gs.data_ptr(),
+                          y.data_ptr(), m, k, n, g, int(trans_rhs), _capi.RD_DTYPE_BF16,
+                          ctypes.byref(plan) if plan is not None else None, ws.data_ptr(), ws.numel())
+    torch.cuda.synchronize()
+    return rc
+
+
+@pytest.mark.parametrize("fill_in", [1.0, 0.5, 0.0])
+def test_every_output_element_is_written(fill_in):
+    """The output buffer arrives uninitialised (gpu_ragged_dot.py:210): poison it and require every element to be
+    overwritten - including when every group is empty, which the reference leaves undefined (:157)."""
+    print("poison fill_in", fill_in, flush=True)
+    m, k, n, g = 300, 128, 136, 7
+    lhs, rhs, _, gs, target_m = util.make_case(11, m, k, n, g, fill_in, True)
+    for plan in (None, _capi.Plan(-1, 0, 64)):
+        y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        assert _raw_gmm(util.bf16_dev(lhs), util.bf16_dev(rhs), torch.from_numpy(gs).cuda(), y, plan=plan) == 0
+        y = util.to_np(y)
+        assert not np.isnan(y).any()
+        util.assert_close_rows(y, oracle.gmm(lhs, rhs, gs), target_m, util.BF16_EPS, "y")
+        assert not np.any(y[target_m:])
+
+
+def test_group_sizes_past_m_are_clipped():
+    """sum(group_sizes) > m is out-of-bounds in the reference; here rows >= m are never touched."""
+    print("clip", flush=True)
+    m, k, n, g = 100, 64, 72, 4
+    lhs, rhs, _, _, _ = util.make_case(2, m, k, n, g, 1.0, True)
+    gs = np.array([40, 40, 40, 40], np.int32)
+    guard = torch.full((m + 64, n), 7.0, dtype=torch.bfloat16, device="cuda")
+    y = guard[:m]
+    assert _raw_gmm(util.bf16_dev(lhs), util.bf16_dev(rhs), torch.from_numpy(gs).cuda(), y) == 0
+    assert torch.all(guard[m:] == 7.0)
+    clipped = np.array([40, 40, 20, 0], np.int32)
+    util.assert_close_rows(util.to_np(y), oracle.gmm(lhs, rhs, clipped), m, util.BF16_EPS, "clipped y")
+
+
+def test_linearity_and_group_locality():
+    """Size-independent properties: scaling x by 2 scales y by exactly 2 (power of two in bf16); changing one
+    group's weights changes only that group's rows."""
+    print("linearity", flush=True)
+    m, k, n, g = 1024, 512, 768, 8
+    lhs, rhs, _, gs, _ = util.make_case(4, m, k, n, g, 1.0, True, scale_rhs=True)
+    x, A, gs_t = util.bf16_dev(lhs), util.bf16_dev(rhs), torch.from_numpy(gs)
+    y1 = rd.gmm(x, A, gs_t)
+    y2 = rd.gmm(x * 2, A, gs_t)
+    assert torch.equal(y2.float(), y1.float() * 2)
+    A2 = A.clone()
+    A2[3] = -A2[3]
+    y3 = rd.gmm(x, A2, gs_t)
+    off = np.concatenate([[0], np.cumsum(gs)])
+    same = torch.ones(m, dtype=torch.bool)
+    same[off[3]:off[4]] = False
+    assert torch.equal(y3[same.cuda()], y1[same.cuda()])
+    assert torch.equal(y3[off[3]:off[4]].float(), -y1[off[3]:off[4]].float())
