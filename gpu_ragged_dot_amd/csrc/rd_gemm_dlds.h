@@ -1,0 +1,251 @@
+// The large-tile GEMM core: HBM -> LDS without a stop in registers (buffer_load_dwordx4 ... lds), STAGES-deep ring of
+// K-slabs in LDS, one barrier per K-step.  Same contract as gemm_tile() in rd_gemm_tile.h; used for the tall tiles
+// that carry the compute-bound shapes.  Needs 16-byte row pitches.
+//
+// LDS layout.  A wave-wide direct load deposits 64 x 16 B contiguously, so rows cannot be padded; bank conflicts are
+// avoided by permuting which 16-byte chunk of a row each lane fetches (an XOR on the chunk index), undone by the
+// matrix-core fragment reads:
+//   K-major slab  [rows][BK]   : chunk c of row r sits at chunk c ^ ((r >> 1) & 7)        (BK = 64, 128-byte rows)
+//                                                       or c ^ ((r >> 2) & 3)              (BK = 32,  64-byte rows)
+//   MN-major slab [BK][rows]   : chunk c of contraction row kk sits at chunk c ^ ((kk & 3) << 2)
+// so that the 16 rows of a 128-bit fragment read, and the 4 rows of a transposing 64-bit read, fall into different
+// bank groups.
+#pragma once
+#include "rd_common.h"
+
+namespace rd {
+
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, bool A_KMAJOR_, bool B_KMAJOR_, int STAGES_>
+struct DldsCfg {
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
+  static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = true, DLDS = true;
+  static constexpr int NW = WAVES_M * WAVES_N;
+  static constexpr int NT = 64 * NW;
+  static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  static constexpr int TM = WM / 32, TN = WN / 32;
+  static constexpr int KSTEPS = BK / 16;
+  static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
+  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+  static_assert(BK == 64 || BK == 32, "contraction slab");
+  static_assert(BM % 128 == 0 && BN % 128 == 0, "direct-to-LDS tiles are at least 128 wide");
+  static_assert(BM % (32 * WAVES_M) == 0 && BN % (32 * WAVES_N) == 0, "tile shape");
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+};
+
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+
+constexpr int kBufferFlags = 0x00020000;   // raw buffer, 32-bit data format
+constexpr int kOobOffset = 0x7ffffff0;     // byte offset past any buffer: the load returns zeros
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is 6 bits");
+  __builtin_amdgcn_s_waitcnt((N & 0xf) | ((N >> 4) << 14) | (0x7 << 4) | (0xf << 8));
+}
+
+// One operand's slab loader: which 16 bytes each lane fetches for each of its wave's load instructions.
+template <int T, int BK, int NW, bool KMAJOR>
+struct DldsLoader {
+  static constexpr int ROW_BYTES = KMAJOR ? BK * 2 : T * 2;
+  static constexpr int RPI = 1024 / ROW_BYTES;   // slab rows per wave-wide load
+  static constexpr int CPR = ROW_BYTES / 16;     // 16-byte chunks per slab row
+  static constexpr int ROWS = KMAJOR ? T : BK;
+  static constexpr int INSTR = ROWS / RPI;       // wave-wide loads per slab
+  static constexpr int PER = INSTR / NW;         // of which each wave issues
+  static_assert(INSTR % NW == 0 && PER >= 1, "slab does not split evenly over the waves");
+  static_assert(!KMAJOR || (NW * RPI) % 16 == 0, "the chunk permutation must repeat from one load slot to the next");
+
+  const bf16_bits* base;  // advances with the K loop
+  int records;            // bytes still addressable from base
+  int step_bytes;         // K-step advance of base in bytes
+  int voff[PER];          // per-lane byte offset of each load
+  int kcol;               // K-major: contraction offset (elements) of this lane's chunk, for the tail predicate
+
+  __device__ __forceinline__ void init(const bf16_bits* p, int ld, int lim, int klen, int wave, int lane) {
+    base = p;
+    if (KMAJOR) {
+      records = ((lim - 1) * ld + klen) * 2;
+      step_bytes = BK * 2;
+    } else {
+      records = ((klen - 1) * ld + lim) * 2;
+      step_bytes = BK * ld * 2;
+    }
+    kcol = 0;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int t = wave + NW * j;
+      const int r = t * RPI + lane / CPR;
+      const int pchunk = lane % CPR;
+      if (KMAJOR) {
+        const int c = pchunk ^ (BK == 64 ? ((r >> 1) & 7) : ((r >> 2) & 3));
+        voff[j] = (imin(r, lim - 1) * ld + c * 8) * 2;
+        kcol = c * 8;  // identical for every j: r advances by a multiple of 16 rows per instruction slot
+      } else {
+        const int c = pchunk ^ ((r & 3) << 2);
+        voff[j] = (r * ld + imin(c * 8, lim - 8)) * 2;
+      }
+    }
+  }
+
+  // Issue this wave's loads of the current slab into `lds` (byte address of the operand's region in one stage).
+  // TAIL: the slab runs past the contraction length.
+  template <bool TAIL>
+  __device__ __forceinline__ void issue(unsigned char* lds, int wave, int k0, int klen) const {
+    __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, __builtin_amdgcn_readfirstlane(records), kBufferFlags);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      int off = voff[j];
+      if (TAIL && KMAJOR && k0 + kcol >= klen) off = kOobOffset;  // MN-major tails are out of `records` by themselves
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(lds + (wave + NW * j) * 1024), 16, off, 0, 0, 0);
+    }
+  }
+
+  __device__ __forceinline__ void advance() {
+    base = reinterpret_cast<const bf16_bits*>(reinterpret_cast<const unsigned char*>(base) + step_bytes);
+    records -= step_bytes;  // stays positive for every slab that is issued
+  }
+};
+
+// Per-lane LDS byte offsets for the matrix-core fragment reads of one operand.
+template <int T, int BK, int TILES, bool KMAJOR>
+struct DldsFragReader {
+  static constexpr int ROW_BYTES = KMAJOR ? BK * 2 : T * 2;
+  static constexpr int KSTEPS = BK / 16;
+  static constexpr int NADDR = KMAJOR ? KSTEPS : TILES;
+  int addr[NADDR];
+
+  __device__ __forceinline__ void init(int wave_idx0, int lane) {
+    if (KMAJOR) {
+      const int r = lane & 31;
+      const int sw = BK == 64 ? ((r >> 1) & 7) : ((r >> 2) & 3);
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks)
+        addr[ks] = (wave_idx0 + r) * ROW_BYTES + (((ks * 2 + (lane >> 5)) ^ sw) << 4);
+    } else {
+      const int q = lane >> 4, i = lane & 15;
+      const int row = 8 * (q >> 1) + (i >> 2);
+      const int s = (i >> 2) & 3;
+      const int low = 2 * (q & 1) + ((i & 3) >> 1);
+#pragma unroll
+      for (int j = 0; j < TILES; ++j) {
+        const int tile = (wave_idx0 >> 5) + j;
+        addr[j] = row * ROW_BYTES + ((4 * (tile ^ s) + low) << 4) + (i & 1) * 8;
+      }
+    }
+  }
+
+  __device__ __forceinline__ bf16x8_t read(const unsigned char* region, int tile, int ks) const {
+    if (KMAJOR) {
+      return *reinterpret_cast<const bf16x8_t*>(region + addr[ks] + tile * 32 * ROW_BYTES);
+    } else {
+      typedef __attribute__((address_space(3))) s16x4_t* lds_v4_ptr;
+      const unsigned char* p = region + addr[tile] + ks * 16 * ROW_BYTES;
+      s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_ptr)(p));
+      s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_ptr)(p + 4 * ROW_BYTES));
+      s16x8_t v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      return __builtin_bit_cast(bf16x8_t, v);
+    }
+  }
+};
+
+template <class C>
+__device__ __forceinline__ void gemm_tile_dlds(const bf16_bits* __restrict__ Ap, int lda, int a_lim,
+                                               const bf16_bits* __restrict__ Bp, int ldb, int b_lim, int klen,
+                                               bf16_bits* __restrict__ Op, int ldo, bf16_bits* smem_) {
+  unsigned char* smem = reinterpret_cast<unsigned char*>(smem_);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;
+
+  typedef DldsLoader<C::BM, C::BK, C::NW, C::A_KMAJOR> LdA;
+  typedef DldsLoader<C::BN, C::BK, C::NW, C::B_KMAJOR> LdB;
+  LdA la; LdB lb;
+  la.init(Ap, lda, a_lim, klen, wave, lane);
+  lb.init(Bp, ldb, b_lim, klen, wave, lane);
+  DldsFragReader<C::BM, C::BK, C::TM, C::A_KMAJOR> fra;
+  DldsFragReader<C::BN, C::BK, C::TN, C::B_KMAJOR> frb;
+  fra.init(wm * C::WM, lane);
+  frb.init(wn * C::WN, lane);
+
+  f32x16_t acc[C::TM][C::TN];
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  const int nk = (klen + C::BK - 1) / C::BK;
+  constexpr int L = LdA::PER + LdB::PER;  // loads per thread per K-step
+
+  auto issue_step = [&](int step) {
+    unsigned char* st = smem + (step % C::STAGES) * C::STAGE_BYTES;
+    const int k0 = step * C::BK;
+    if (k0 + C::BK <= klen) {
+      la.template issue<false>(st, wave, k0, klen);
+      lb.template issue<false>(st + C::A_BYTES, wave, k0, klen);
+    } else {
+      la.template issue<true>(st, wave, k0, klen);
+      lb.template issue<true>(st + C::A_BYTES, wave, k0, klen);
+    }
+    la.advance();
+    lb.advance();
+  };
+
+  // prologue: STAGES-1 slabs in flight
+#pragma unroll
+  for (int s = 0; s < C::STAGES - 1; ++s)
+    if (s < nk) issue_step(s);
+
+  for (int kt = 0; kt < nk; ++kt) {
+    // Slab kt must have landed; the STAGES-2 younger ones may still be in flight.  Near the end fewer loads were
+    // issued after slab kt than that, so wait for everything.
+    if (kt + C::STAGES - 2 < nk) wait_vmcnt<(C::STAGES - 2) * L>(); else wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();  // every wave's part of slab kt is in LDS, and slab kt-1 is no longer being read
+    if (kt + C::STAGES - 1 < nk) issue_step(kt + C::STAGES - 1);
+
+    const unsigned char* ra = smem + (kt % C::STAGES) * C::STAGE_BYTES;
+    const unsigned char* rb = ra + C::A_BYTES;
+    // Fragments for K-substep ks+1 are fetched from LDS while the matrix core works on substep ks.
+    bf16x8_t fa[2][C::TM], fb[2][C::TN];
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i) fa[0][i] = fra.read(ra, i, 0);
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) fb[0][j] = frb.read(rb, j, 0);
+#pragma unroll
+    for (int ks = 0; ks < C::KSTEPS; ++ks) {
+      const int cur = ks & 1, nxt = cur ^ 1;
+      if (ks + 1 < C::KSTEPS) {
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i) fa[nxt][i] = fra.read(ra, i, ks + 1);
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) fb[nxt][j] = frb.read(rb, j, ks + 1);
+      }
+      // Keep the compiler from sinking those reads back below the matrix-core work they are meant to overlap.
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) {
+      const int col = wn * C::WN + j * 32 + (lane & 31);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = wm * C::WM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        if (row < a_lim && col < b_lim) Op[(size_t)row * ldo + col] = f32_to_bf16(acc[i][j][v]);
+      }
+    }
+  }
+}
+
+}  // namespace rd

@@ -1,6 +1,7 @@
 // Grouped-GEMM kernels built on gemm_tile(): launch-index -> tile mapping, group lookup through the scheduling
 // map, tail / empty-group zeroing.
 #pragma once
+#include "rd_gemm_dlds.h"
 #include "rd_gemm_tile.h"
 
 namespace rd {
@@ -33,6 +34,16 @@ struct TgmmArgs {
   int group_m;
 };
 
+// A value every lane holds identically, moved to a scalar register.
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+template <class C>
+__device__ __forceinline__ void run_tile(const bf16_bits* Ap, int lda, int a_lim, const bf16_bits* Bp, int ldb,
+                                         int b_lim, int klen, bf16_bits* Op, int ldo, bf16_bits* smem) {
+  if constexpr (C::DLDS) gemm_tile_dlds<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
+  else gemm_tile<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
+}
+
 // Walk tiles in bands of `group_m` rows: consecutive ids share B columns / A rows so that the ~32 tiles one XCD
 // has in flight re-use each other's operands out of its L2.
 __device__ __forceinline__ void band_walk(int id, int rows, int cols, int group_m, int& ri, int& cj) {
@@ -52,26 +63,27 @@ __global__ __launch_bounds__(C::NT) void gmm_kernel(GmmArgs p) {
   int mi, nj;
   band_walk(id, p.U, p.n_tiles, p.group_m, mi, nj);
 
-  const int total = imin(*p.total_tiles, p.U);
+  // Everything read through the map is the same for the whole work-group: pin it to scalar registers.
+  const int total = imin(uniform(*p.total_tiles), p.U);
   const int col0 = nj * C::BN;
   const int cols = imin(C::BN, p.n - col0);
 
   if (mi < total) {
-    const int gi = p.tile2group[mi];
-    const int it = p.tile2it[mi];
-    const int row0 = p.group_offsets[gi] + it * C::BM;
-    int rows = imin(C::BM, p.group_sizes[gi] - it * C::BM);
+    const int gi = uniform(p.tile2group[mi]);
+    const int it = uniform(p.tile2it[mi]);
+    const int row0 = uniform(p.group_offsets[gi]) + it * C::BM;
+    int rows = imin(C::BM, uniform(p.group_sizes[gi]) - it * C::BM);
     rows = imin(rows, p.m - row0);  // group_sizes summing past m: never touch rows >= m
     if (rows <= 0 || row0 < 0) return;
     const bf16_bits* Ap = p.x + (size_t)row0 * p.k;
     const bf16_bits* Bp = TRANS_RHS ? p.A + (size_t)gi * p.n * p.k + (size_t)col0 * p.k
                                     : p.A + (size_t)gi * p.k * p.n + col0;
     bf16_bits* Op = p.y + (size_t)row0 * p.n + col0;
-    gemm_tile<C>(Ap, p.k, rows, Bp, TRANS_RHS ? p.k : p.n, cols, p.k, Op, p.n, smem);
+    run_tile<C>(Ap, p.k, rows, Bp, TRANS_RHS ? p.k : p.n, cols, p.k, Op, p.n, smem);
   } else {
     // Rows past sum(group_sizes) are defined to be zero.  The map never uses more than
     // U - ceil(tail / BM) entries, so the unused tile slots cover the tail.
-    long long s = (long long)p.group_offsets[p.g - 1] + p.group_sizes[p.g - 1];
+    long long s = (long long)uniform(p.group_offsets[p.g - 1]) + uniform(p.group_sizes[p.g - 1]);
     if (s < 0) s = 0;
     const long long r0 = s + (long long)(mi - total) * C::BM;
     if (r0 >= p.m) return;
@@ -94,8 +106,8 @@ __global__ __launch_bounds__(C::NT) void tgmm_kernel(TgmmArgs p) {
   const int krows = imin(C::BM, p.k - kk0), cols = imin(C::BN, p.n - col0);
   bf16_bits* Op = p.dA + (size_t)gi * p.k * p.n + (size_t)kk0 * p.n + col0;
 
-  const int row0 = p.group_offsets[gi];
-  int rows = p.group_sizes[gi];
+  const int row0 = uniform(p.group_offsets[gi]);
+  int rows = uniform(p.group_sizes[gi]);
   rows = imin(rows, p.m - row0);
   if (rows <= 0 || row0 < 0) {  // empty group: its slice of dA is zero
     zero_tile<C::NT, C::VEC>(Op, p.n, krows, cols);
@@ -103,7 +115,7 @@ __global__ __launch_bounds__(C::NT) void tgmm_kernel(TgmmArgs p) {
   }
   const bf16_bits* Ap = p.x + (size_t)row0 * p.k + kk0;
   const bf16_bits* Bp = p.dy + (size_t)row0 * p.n + col0;
-  gemm_tile<C>(Ap, p.k, krows, Bp, p.n, cols, rows, Op, p.n, smem);
+  run_tile<C>(Ap, p.k, krows, Bp, p.n, cols, rows, Op, p.n, smem);
 }
 
 // ---- host-side launchers, one set per compiled tile shape -------------------------------------------------------
@@ -115,6 +127,8 @@ struct TileVariant {
   const char* name;
   int bm, bn, bk, waves_m, waves_n;
   int vec;  // 1: needs k % 8 == 0 and n % 8 == 0 (16-byte row pitches); 0: any shape
+  int dlds;    // 1: direct-to-LDS core (byte extents of one tile's operand window must stay below 2 GiB)
+  int stages;  // LDS ring depth
   gmm_launch_fn gmm_nn, gmm_nt;
   tgmm_launch_fn tgmm;
 };
