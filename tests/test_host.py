@@ -1,0 +1,127 @@
+"""CPU-side checks of the host layer: the C ABI library loads and exports every symbol the header declares, argument
+validation returns error codes (no device work is launched), and the planner follows the reference's block rules."""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from gpu_ragged_dot_amd import _capi, planner
+from oracle import ragged_dot_oracle as oracle
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "ragged_dot_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(rd_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_functions()
+    assert len(names) >= 11
+    lib = ctypes.CDLL(_capi.LIB_PATH)
+    for name in names:
+        assert hasattr(lib, name), f"{name} declared in include/ragged_dot_hip.h but not exported"
+    assert sorted(_capi.EXPORTS) == names, "the ctypes binding must cover exactly what the header declares"
+    assert _capi.lib.rd_abi_version() == 1
+
+
+def test_variant_table():
+    vs = _capi.variants()
+    assert len(vs) >= 2
+    names = [v.name.decode() for v in vs]
+    assert len(set(names)) == len(names)
+    assert any(v.vec == 0 for v in vs), "an any-shape variant must exist for pitches that are not 16-byte multiples"
+    for v in vs:
+        assert v.tile_m % (32 * v.waves_m) == 0 and v.tile_n % (32 * v.waves_n) == 0 and v.tile_k % 16 == 0
+        if v.direct_to_lds:
+            assert v.vec == 1 and v.stages * (v.tile_m + v.tile_n) * v.tile_k * 2 <= 160 * 1024
+
+
+def test_argument_validation_returns_codes():
+    lib = _capi.lib
+    one = ctypes.c_void_p(16)  # never dereferenced: validation fails first
+    rc = lib.rd_gmm(None, one, one, one, one, 8, 8, 8, 0, 0, _capi.RD_DTYPE_BF16, None, one, 1 << 20)
+    assert rc == _capi.RD_ERR_INVALID_ARGUMENT and b"g=0" in lib.rd_last_error()
+    rc = lib.rd_gmm(None, one, one, one, one, -1, 8, 8, 2, 0, _capi.RD_DTYPE_BF16, None, one, 1 << 20)
+    assert rc == _capi.RD_ERR_INVALID_ARGUMENT
+    rc = lib.rd_gmm(None, one, one, None, one, 8, 8, 8, 2, 0, _capi.RD_DTYPE_BF16, None, one, 1 << 20)
+    assert rc == _capi.RD_ERR_INVALID_ARGUMENT and b"null" in lib.rd_last_error()
+    rc = lib.rd_gmm(None, one, one, one, one, 8, 8, 8, 2, 0, 7, None, one, 1 << 20)
+    assert rc == _capi.RD_ERR_INVALID_ARGUMENT
+    rc = lib.rd_gmm(None, one, one, one, one, 8, 8, 8, 2, 0, _capi.RD_DTYPE_F32, None, one, 1 << 20)
+    assert rc == _capi.RD_ERR_UNSUPPORTED
+    rc = lib.rd_tgmm(None, one, one, one, one, 8, 8, 8, 0, _capi.RD_DTYPE_BF16, None, one, 1 << 20)
+    assert rc == _capi.RD_ERR_INVALID_ARGUMENT
+    rc = lib.rd_sched_map(None, one, 0, 8, 8, one, one, one, one)
+    assert rc == _capi.RD_ERR_INVALID_ARGUMENT
+    rc = lib.rd_sched_map(None, one, 4, 8, 0, one, one, one, one)
+    assert rc == _capi.RD_ERR_INVALID_ARGUMENT
+    with pytest.raises(_capi.RaggedDotError):
+        _capi.check(rc)
+    assert lib.rd_get_variant(10 ** 6, ctypes.byref(_capi.VariantInfo())) == _capi.RD_ERR_INVALID_ARGUMENT
+    # a plan that names a missing variant, a too-small workspace, a vector variant on an unaligned shape
+    plan = _capi.Plan(10 ** 6, 0, 0)
+    rc = lib.rd_gmm(None, one, one, one, one, 8, 8, 8, 2, 0, _capi.RD_DTYPE_BF16, ctypes.byref(plan), one, 1 << 20)
+    assert rc == _capi.RD_ERR_INVALID_ARGUMENT
+    rc = lib.rd_gmm(None, one, one, one, one, 64, 64, 64, 2, 0, _capi.RD_DTYPE_BF16, None, one, 8)
+    assert rc == _capi.RD_ERR_WORKSPACE
+    vec_id = next(v.id for v in _capi.variants() if v.vec)
+    plan = _capi.Plan(vec_id, 0, 0)
+    rc = lib.rd_gmm(None, one, one, one, one, 64, 58, 77, 2, 0, _capi.RD_DTYPE_BF16, ctypes.byref(plan), one, 1 << 20)
+    assert rc == _capi.RD_ERR_UNSUPPORTED
+
+
+def test_workspace_and_map_sizes():
+    lib = _capi.lib
+    assert lib.rd_sched_map_len(16384, 8, 512) == 40  # U of the Mixtral config at the reference's chunk
+    assert lib.rd_sched_map_len(64, 128, 512) == 129
+    assert lib.rd_sched_map_len(0, 3, 8) == 3
+    for m, g in ((16384, 8), (32768, 256), (64, 128), (0, 1)):
+        need = lib.rd_gmm_workspace_bytes(m, g, None)
+        for v in _capi.variants():
+            U = -(-m // v.tile_m) + g
+            assert need >= (g + 2 * U + 1) * 4
+        assert lib.rd_tgmm_workspace_bytes(m, g, None) >= (g + 2 * (g + 1) + 1) * 4
+
+
+def test_planner_block_rules_match_the_oracle():
+    for args in ((64, 64, 64, 16384, 4096, 14336), (16, 16, 16, 171, 58, 77), (8, 8, 8, 100, 100, 100),
+                 (256, 256, 256, 5, 40, 9), (32, 64, 16, 128, 512, 64)):
+        assert planner.normalize_gmm_blocks(*args) == oracle.gmm_block_sizes(*args)
+        assert planner.normalize_tgmm_blocks(*args) == oracle.tgmm_block_sizes(*args)
+
+
+def test_planner_choices():
+    vs = {v.id: v for v in _capi.variants()}
+    p = planner.select_plan(_capi.OP_GMM, 171, 58, 77, 8)
+    assert vs[p.variant].vec == 0 and p.decode_nb == 0  # odd pitches -> any-shape variant
+    p = planner.select_plan(_capi.OP_GMM, 64, 2048, 768, 128)
+    assert p.decode_nb > 0  # a few rows per expert -> streaming kernel
+    p = planner.select_plan(_capi.OP_GMM_TRANS, 64, 2048, 768, 128)
+    assert p.decode_nb == 0
+    p = planner.select_plan(_capi.OP_GMM, 16384, 4096, 14336, 8)
+    assert vs[p.variant].tile_m == 256 and vs[p.variant].tile_n == 256
+    p = planner.select_plan(_capi.OP_GMM, 16384, 4096, 14336, 8, block_m=128, block_k=64, block_n=128)
+    assert (vs[p.variant].tile_m, vs[p.variant].tile_n) == (128, 128)  # explicit request -> nearest compiled shape
+
+
+def test_cpu_tensors_are_rejected_loudly():
+    import gpu_ragged_dot_amd as rd
+
+    x = torch.zeros(8, 8, dtype=torch.bfloat16)
+    A = torch.zeros(2, 8, 8, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        rd.ragged_dot(x, A, torch.tensor([4, 4], dtype=torch.int32))
+    with pytest.raises(NotImplementedError):
+        rd.ragged_dot(x, A, torch.tensor([4, 4], dtype=torch.int32), interpret=True)
+    with pytest.raises(AssertionError):
+        rd.ragged_dot(x, A[0], torch.tensor([4, 4], dtype=torch.int32))  # gpu_ragged_dot.py:188
+    with pytest.raises(AssertionError):
+        rd.ragged_dot(x, A, torch.tensor([4, 2, 2], dtype=torch.int32))  # gpu_ragged_dot.py:189
+    with pytest.raises(AssertionError):
+        rd.tgmm(x, torch.zeros(9, 8, dtype=torch.bfloat16), torch.tensor([4, 4], dtype=torch.int32))  # :304
