@@ -13,12 +13,19 @@
 #pragma once
 #include "rd_common.h"
 
+// Hook for timing experiments: a build may define RD_MARK(id) to record a timestamp at each pipeline phase.
+#ifndef RD_MARK
+#define RD_MARK(id)
+#define RD_MARK_DECL
+#endif
+
 namespace rd {
 
-template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, bool A_KMAJOR_, bool B_KMAJOR_, int STAGES_>
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, bool A_KMAJOR_, bool B_KMAJOR_, int STAGES_,
+          bool PINGPONG_ = false>
 struct DldsCfg {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
-  static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = true, DLDS = true;
+  static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = true, DLDS = true, PINGPONG = PINGPONG_;
   static constexpr int NW = WAVES_M * WAVES_N;
   static constexpr int NT = 64 * NW;
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
@@ -26,11 +33,17 @@ struct DldsCfg {
   static constexpr int KSTEPS = BK / 16;
   static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+  // The epilogue re-uses LDS to turn accumulators into row-contiguous 16-byte stores: one [WM][WN] bf16 patch per
+  // wave, rows padded by 16 bytes.
+  static constexpr int EPI_PITCH = WN * 2 + 16;
+  static constexpr int EPI_BYTES = NW * WM * EPI_PITCH;
+  static constexpr int RING_BYTES = STAGES * STAGE_BYTES;
+  static constexpr int LDS_BYTES = RING_BYTES > EPI_BYTES ? RING_BYTES : EPI_BYTES;
   static_assert(BK == 64 || BK == 32, "contraction slab");
   static_assert(BM % 128 == 0 && BN % 128 == 0, "direct-to-LDS tiles are at least 128 wide");
   static_assert(BM % (32 * WAVES_M) == 0 && BN % (32 * WAVES_N) == 0, "tile shape");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+  static_assert(!PINGPONG || (NW == 8 && WAVES_M == 2 && STAGES >= 2), "ping-pong runs two groups of four waves");
 };
 
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
@@ -88,18 +101,18 @@ struct DldsLoader {
     }
   }
 
-  // Issue this wave's loads of the current slab into `lds` (byte address of the operand's region in one stage).
+  __device__ __forceinline__ __amdgpu_buffer_rsrc_t resource() const {
+    return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, __builtin_amdgcn_readfirstlane(records), kBufferFlags);
+  }
+
+  // Issue load j of this wave for the current slab into `lds` (byte address of the operand's region in one stage).
   // TAIL: the slab runs past the contraction length.
   template <bool TAIL>
-  __device__ __forceinline__ void issue(unsigned char* lds, int wave, int k0, int klen) const {
-    __amdgpu_buffer_rsrc_t rsrc =
-        __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, __builtin_amdgcn_readfirstlane(records), kBufferFlags);
-#pragma unroll
-    for (int j = 0; j < PER; ++j) {
-      int off = voff[j];
-      if (TAIL && KMAJOR && k0 + kcol >= klen) off = kOobOffset;  // MN-major tails are out of `records` by themselves
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(lds + (wave + NW * j) * 1024), 16, off, 0, 0, 0);
-    }
+  __device__ __forceinline__ void issue(__amdgpu_buffer_rsrc_t rsrc, unsigned char* lds, int wave, int j, int k0,
+                                        int klen) const {
+    int off = voff[j];
+    if (TAIL && KMAJOR && k0 + kcol >= klen) off = kOobOffset;  // MN-major tails are out of `records` by themselves
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(lds + (wave + NW * j) * 1024), 16, off, 0, 0, 0);
   }
 
   __device__ __forceinline__ void advance() {
@@ -150,10 +163,47 @@ struct DldsFragReader {
   }
 };
 
+// Epilogue shared by the direct-to-LDS cores.  The matrix-core calls pass the B fragment as first operand, so the
+// accumulators hold transposed 32x32 blocks: register v of lane l is C[l & 31][8*(v>>2) + 4*(l>>5) + (v&3)], i.e. four
+// consecutive columns of one row per register quad.  Each wave drops its [WM][WN] patch into its own LDS area as bf16
+// (8-byte writes), then streams it out with 16-byte loads/stores that cover whole 128-byte lines of the output rows.
+// Only the wave itself touches its area, so no work-group barrier is needed in between.
+template <class C>
+__device__ __forceinline__ void store_accumulators(const f32x16_t (&acc)[C::TM][C::TN], int wm, int wn, int wave,
+                                                   int lane, int a_lim, int b_lim, bf16_bits* __restrict__ Op, int ldo,
+                                                   unsigned char* smem) {
+  unsigned char* st = smem + wave * (C::WM * C::EPI_PITCH);
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int row = i * 32 + (lane & 31);
+        const int col = j * 32 + 8 * g + 4 * (lane >> 5);
+        u32x2_t w;
+        w[0] = pack_bf16x2(acc[i][j][4 * g + 0], acc[i][j][4 * g + 1]);
+        w[1] = pack_bf16x2(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+        *reinterpret_cast<u32x2_t*>(st + row * C::EPI_PITCH + col * 2) = w;
+      }
+  constexpr int CPR = C::WN / 8;        // 16-byte chunks per patch row
+  constexpr int ROWS_PER = 64 / CPR;    // patch rows per wave-wide store
+  const int chunk = lane % CPR, r0 = lane / CPR;
+  const int gcol = wn * C::WN + chunk * 8;
+#pragma unroll
+  for (int t = 0; t < C::WM / ROWS_PER; ++t) {
+    const int row = t * ROWS_PER + r0;
+    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(st + row * C::EPI_PITCH + chunk * 16);
+    const int grow = wm * C::WM + row;
+    if (grow < a_lim && gcol < b_lim) *reinterpret_cast<u32x4_t*>(Op + (size_t)grow * ldo + gcol) = v;
+  }
+}
+
 template <class C>
 __device__ __forceinline__ void gemm_tile_dlds(const bf16_bits* __restrict__ Ap, int lda, int a_lim,
                                                const bf16_bits* __restrict__ Bp, int ldb, int b_lim, int klen,
                                                bf16_bits* __restrict__ Op, int ldo, bf16_bits* smem_) {
+  RD_MARK_DECL;
   unsigned char* smem = reinterpret_cast<unsigned char*>(smem_);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -180,35 +230,44 @@ __device__ __forceinline__ void gemm_tile_dlds(const bf16_bits* __restrict__ Ap,
   const int nk = (klen + C::BK - 1) / C::BK;
   constexpr int L = LdA::PER + LdB::PER;  // loads per thread per K-step
 
-  auto issue_step = [&](int step) {
+  // Loads [first, first + count) of slab `step` (the A loads come first in the numbering, then the B loads).
+  auto issue_loads = [&](int step, int first, int count) {
     unsigned char* st = smem + (step % C::STAGES) * C::STAGE_BYTES;
     const int k0 = step * C::BK;
-    if (k0 + C::BK <= klen) {
-      la.template issue<false>(st, wave, k0, klen);
-      lb.template issue<false>(st + C::A_BYTES, wave, k0, klen);
-    } else {
-      la.template issue<true>(st, wave, k0, klen);
-      lb.template issue<true>(st + C::A_BYTES, wave, k0, klen);
+    const bool tail = k0 + C::BK > klen;
+    __amdgpu_buffer_rsrc_t ra_ = la.resource(), rb_ = lb.resource();
+#pragma unroll
+    for (int q = first; q < first + count; ++q) {
+      if (q < LdA::PER) {
+        if (tail) la.template issue<true>(ra_, st, wave, q, k0, klen);
+        else la.template issue<false>(ra_, st, wave, q, k0, klen);
+      } else {
+        if (tail) lb.template issue<true>(rb_, st + C::A_BYTES, wave, q - LdA::PER, k0, klen);
+        else lb.template issue<false>(rb_, st + C::A_BYTES, wave, q - LdA::PER, k0, klen);
+      }
     }
-    la.advance();
-    lb.advance();
   };
 
   // prologue: STAGES-1 slabs in flight
 #pragma unroll
   for (int s = 0; s < C::STAGES - 1; ++s)
-    if (s < nk) issue_step(s);
+    if (s < nk) { issue_loads(s, 0, L); la.advance(); lb.advance(); }
 
   for (int kt = 0; kt < nk; ++kt) {
+    RD_MARK(0);
     // Slab kt must have landed; the STAGES-2 younger ones may still be in flight.  Near the end fewer loads were
     // issued after slab kt than that, so wait for everything.
     if (kt + C::STAGES - 2 < nk) wait_vmcnt<(C::STAGES - 2) * L>(); else wait_vmcnt<0>();
+    RD_MARK(1);
     __builtin_amdgcn_s_barrier();  // every wave's part of slab kt is in LDS, and slab kt-1 is no longer being read
-    if (kt + C::STAGES - 1 < nk) issue_step(kt + C::STAGES - 1);
+    RD_MARK(2);
+    const bool more = kt + C::STAGES - 1 < nk;
 
     const unsigned char* ra = smem + (kt % C::STAGES) * C::STAGE_BYTES;
     const unsigned char* rb = ra + C::A_BYTES;
-    // Fragments for K-substep ks+1 are fetched from LDS while the matrix core works on substep ks.
+    // Fragments for K-substep ks+1 are fetched from LDS while the matrix core works on substep ks, and the loads of
+    // the slab STAGES-1 steps ahead are issued a few at a time between the substeps: the memory pipeline then works
+    // through them in the shadow of the matrix-core instructions instead of stalling every wave at once.
     bf16x8_t fa[2][C::TM], fb[2][C::TN];
 #pragma unroll
     for (int i = 0; i < C::TM; ++i) fa[0][i] = fra.read(ra, i, 0);
@@ -223,29 +282,232 @@ __device__ __forceinline__ void gemm_tile_dlds(const bf16_bits* __restrict__ Ap,
 #pragma unroll
         for (int j = 0; j < C::TN; ++j) fb[nxt][j] = frb.read(rb, j, ks + 1);
       }
-      // Keep the compiler from sinking those reads back below the matrix-core work they are meant to overlap.
+      if (more) {
+        constexpr int lo = 0;
+        const int first = (L * ks) / C::KSTEPS, last = (L * (ks + 1)) / C::KSTEPS;
+        (void)lo;
+        issue_loads(kt + C::STAGES - 1, first, last - first);
+      }
+      // Keep the compiler from sinking those reads and loads below the matrix-core work they are meant to overlap.
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < C::TM; ++i)
 #pragma unroll
         for (int j = 0; j < C::TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
+    if (more) { la.advance(); lb.advance(); }
+    RD_MARK(3);
   }
 
+  __builtin_amdgcn_s_barrier();  // the ring is no longer read by any wave
+  store_accumulators<C>(acc, wm, wn, wave, lane, a_lim, b_lim, Op, ldo, smem);
+}
+
+// Ping-pong schedule.  The eight waves form two groups of four (one wave of each group per SIMD).  A wave alternates
+// between a memory phase (LDS -> registers for one K-slab, plus issuing its share of the direct loads of a later slab)
+// and a compute phase (nothing but matrix-core instructions on registers).  The groups run half a period apart, so on
+// every SIMD one wave always has a full phase of matrix-core work while the other hides all LDS and HBM latency.
+// Work-group barriers separate the phases; the second group passes one extra barrier up front, the first one at the end.
+template <class C>
+__device__ __forceinline__ void gemm_tile_pingpong(const bf16_bits* __restrict__ Ap, int lda, int a_lim,
+                                                   const bf16_bits* __restrict__ Bp, int ldb, int b_lim, int klen,
+                                                   bf16_bits* __restrict__ Op, int ldo, bf16_bits* smem_) {
+  unsigned char* smem = reinterpret_cast<unsigned char*>(smem_);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;  // wm is also the group index
+  const int group = wave >> 2;
+
+  typedef DldsLoader<C::BM, C::BK, C::NW, C::A_KMAJOR> LdA;
+  typedef DldsLoader<C::BN, C::BK, C::NW, C::B_KMAJOR> LdB;
+  LdA la; LdB lb;
+  la.init(Ap, lda, a_lim, klen, wave, lane);
+  lb.init(Bp, ldb, b_lim, klen, wave, lane);
+  DldsFragReader<C::BM, C::BK, C::TM, C::A_KMAJOR> fra;
+  DldsFragReader<C::BN, C::BK, C::TN, C::B_KMAJOR> frb;
+  fra.init(wm * C::WM, lane);
+  frb.init(wn * C::WN, lane);
+
+  f32x16_t acc[C::TM][C::TN];
 #pragma unroll
-  for (int i = 0; i < C::TM; ++i) {
+  for (int i = 0; i < C::TM; ++i)
 #pragma unroll
-    for (int j = 0; j < C::TN; ++j) {
-      const int col = wn * C::WN + j * 32 + (lane & 31);
+    for (int j = 0; j < C::TN; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int row = wm * C::WM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-        if (row < a_lim && col < b_lim) Op[(size_t)row * ldo + col] = f32_to_bf16(acc[i][j][v]);
-      }
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  const int nk = (klen + C::BK - 1) / C::BK;
+  constexpr int L = LdA::PER + LdB::PER;
+
+  auto issue_slab = [&](int step) {
+    unsigned char* st = smem + (step % C::STAGES) * C::STAGE_BYTES;
+    const int k0 = step * C::BK;
+    const bool tail = k0 + C::BK > klen;
+    __amdgpu_buffer_rsrc_t ra_ = la.resource(), rb_ = lb.resource();
+#pragma unroll
+    for (int q = 0; q < LdA::PER; ++q) {
+      if (tail) la.template issue<true>(ra_, st, wave, q, k0, klen);
+      else la.template issue<false>(ra_, st, wave, q, k0, klen);
     }
+#pragma unroll
+    for (int q = 0; q < LdB::PER; ++q) {
+      if (tail) lb.template issue<true>(rb_, st + C::A_BYTES, wave, q, k0, klen);
+      else lb.template issue<false>(rb_, st + C::A_BYTES, wave, q, k0, klen);
+    }
+    la.advance();
+    lb.advance();
+  };
+
+#pragma unroll
+  for (int s = 0; s < C::STAGES - 1; ++s)
+    if (s < nk) issue_slab(s);
+  // slab 0 of every wave must be in LDS before the first memory phase reads it
+  if (C::STAGES - 1 <= nk) wait_vmcnt<(C::STAGES - 2) * L>(); else wait_vmcnt<0>();
+  __builtin_amdgcn_s_barrier();
+  if (group == 1) __builtin_amdgcn_s_barrier();
+
+  for (int kt = 0; kt < nk; ++kt) {
+    // ---- memory phase -------------------------------------------------------------------------------------------
+    const unsigned char* ra = smem + (kt % C::STAGES) * C::STAGE_BYTES;
+    const unsigned char* rb = ra + C::A_BYTES;
+    bf16x8_t fa[C::KSTEPS][C::TM], fb[C::KSTEPS][C::TN];
+#pragma unroll
+    for (int ks = 0; ks < C::KSTEPS; ++ks) {
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i) fa[ks][i] = fra.read(ra, i, ks);
+#pragma unroll
+      for (int j = 0; j < C::TN; ++j) fb[ks][j] = frb.read(rb, j, ks);
+    }
+    // The slot of slab kt-1 is free: both groups finished reading it before the barrier that opened this phase.
+    if (kt + C::STAGES - 1 < nk) issue_slab(kt + C::STAGES - 1);
+    // Before leaving: this wave's share of slab kt+1 has landed (the other group may read it in the very next
+    // interval) and the fragment reads above have returned (the slot they came from may be overwritten next).
+    if (kt + C::STAGES - 1 < nk) wait_vmcnt<(C::STAGES - 2) * L>(); else wait_vmcnt<0>();
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- compute phase ------------------------------------------------------------------------------------------
+    __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+    for (int ks = 0; ks < C::KSTEPS; ++ks)
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
+    __builtin_amdgcn_s_setprio(0);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
   }
+  if (group == 0) __builtin_amdgcn_s_barrier();
+
+  store_accumulators<C>(acc, wm, wn, wave, lane, a_lim, b_lim, Op, ldo, smem);
+}
+
+// Ping-pong on a two-slot ring (room for 64-wide K-slabs, which keep K-major operands on whole 128-byte lines).
+// With only two slots a slab can be requested no earlier than two phases before its first use, so both groups issue
+// their share of slab kt+1 at the start of the same interval: the first group at the head of its memory phase, the
+// second at the head of its compute phase.
+template <class C>
+__device__ __forceinline__ void gemm_tile_pingpong2(const bf16_bits* __restrict__ Ap, int lda, int a_lim,
+                                                    const bf16_bits* __restrict__ Bp, int ldb, int b_lim, int klen,
+                                                    bf16_bits* __restrict__ Op, int ldo, bf16_bits* smem_) {
+  static_assert(C::STAGES == 2, "two-slot ring");
+  unsigned char* smem = reinterpret_cast<unsigned char*>(smem_);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;
+  const int group = wave >> 2;
+
+  typedef DldsLoader<C::BM, C::BK, C::NW, C::A_KMAJOR> LdA;
+  typedef DldsLoader<C::BN, C::BK, C::NW, C::B_KMAJOR> LdB;
+  LdA la; LdB lb;
+  la.init(Ap, lda, a_lim, klen, wave, lane);
+  lb.init(Bp, ldb, b_lim, klen, wave, lane);
+  DldsFragReader<C::BM, C::BK, C::TM, C::A_KMAJOR> fra;
+  DldsFragReader<C::BN, C::BK, C::TN, C::B_KMAJOR> frb;
+  fra.init(wm * C::WM, lane);
+  frb.init(wn * C::WN, lane);
+
+  f32x16_t acc[C::TM][C::TN];
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  const int nk = (klen + C::BK - 1) / C::BK;
+
+  auto issue_slab = [&](int step) {
+    unsigned char* st = smem + (step & 1) * C::STAGE_BYTES;
+    const int k0 = step * C::BK;
+    const bool tail = k0 + C::BK > klen;
+    __amdgpu_buffer_rsrc_t ra_ = la.resource(), rb_ = lb.resource();
+#pragma unroll
+    for (int q = 0; q < LdA::PER; ++q) {
+      if (tail) la.template issue<true>(ra_, st, wave, q, k0, klen);
+      else la.template issue<false>(ra_, st, wave, q, k0, klen);
+    }
+#pragma unroll
+    for (int q = 0; q < LdB::PER; ++q) {
+      if (tail) lb.template issue<true>(rb_, st + C::A_BYTES, wave, q, k0, klen);
+      else lb.template issue<false>(rb_, st + C::A_BYTES, wave, q, k0, klen);
+    }
+    la.advance();
+    lb.advance();
+  };
+
+  if (nk > 0) issue_slab(0);
+  wait_vmcnt<0>();
+  __builtin_amdgcn_s_barrier();
+  if (group == 1) {
+    if (1 < nk) issue_slab(1);
+    __builtin_amdgcn_s_barrier();
+  }
+
+  for (int kt = 0; kt < nk; ++kt) {
+    // ---- memory phase -------------------------------------------------------------------------------------------
+    if (group == 0 && kt + 1 < nk) issue_slab(kt + 1);
+    const unsigned char* ra = smem + (kt & 1) * C::STAGE_BYTES;
+    const unsigned char* rb = ra + C::A_BYTES;
+    bf16x8_t fa[C::KSTEPS][C::TM], fb[C::KSTEPS][C::TN];
+#pragma unroll
+    for (int ks = 0; ks < C::KSTEPS; ++ks) {
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i) fa[ks][i] = fra.read(ra, i, ks);
+#pragma unroll
+      for (int j = 0; j < C::TN; ++j) fb[ks][j] = frb.read(rb, j, ks);
+    }
+    if (group == 1) wait_vmcnt<0>();       // second group's share of slab kt+1 (requested during its last compute phase)
+    __builtin_amdgcn_s_waitcnt(0xc07f);    // lgkmcnt(0): fragments are in registers, the slot may be refilled
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- compute phase ------------------------------------------------------------------------------------------
+    if (group == 1 && kt + 2 < nk) issue_slab(kt + 2);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+    for (int ks = 0; ks < C::KSTEPS; ++ks)
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
+    __builtin_amdgcn_s_setprio(0);
+    if (group == 0) wait_vmcnt<0>();       // first group's share of slab kt+1
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (group == 0) __builtin_amdgcn_s_barrier();
+
+  store_accumulators<C>(acc, wm, wn, wave, lane, a_lim, b_lim, Op, ldo, smem);
 }
 
 }  // namespace rd

@@ -1,5 +1,5 @@
 // One compiled tile shape.  Built once per entry of the variant list in the Makefile, with
-//   -DRD_BM= -DRD_BN= -DRD_BK= -DRD_WAVES_M= -DRD_WAVES_N= -DRD_VEC= -DRD_NAME= [-DRD_DLDS=1 -DRD_STAGES=]
+//   -DRD_BM= -DRD_BN= -DRD_BK= -DRD_WAVES_M= -DRD_WAVES_N= -DRD_VEC= -DRD_NAME= [-DRD_DLDS=1 -DRD_STAGES= -DRD_PINGPONG=1]
 // and exports a getter rd_variant_<name>() for its TileVariant record that the C-ABI file collects.
 #include "rd_kernels.h"
 
@@ -14,12 +14,15 @@
 #ifndef RD_STAGES
 #define RD_STAGES 2
 #endif
+#ifndef RD_PINGPONG
+#define RD_PINGPONG 0
+#endif
 
 namespace rd {
 #if RD_DLDS
-typedef DldsCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, /*A K-major*/ true, /*B K-major*/ false, RD_STAGES> CfgNN;
-typedef DldsCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, true, true, RD_STAGES> CfgNT;
-typedef DldsCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, false, false, RD_STAGES> CfgTN;
+typedef DldsCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, /*A K-major*/ true, /*B K-major*/ false, RD_STAGES, RD_PINGPONG != 0> CfgNN;
+typedef DldsCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, true, true, RD_STAGES, RD_PINGPONG != 0> CfgNT;
+typedef DldsCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, false, false, RD_STAGES, RD_PINGPONG != 0> CfgTN;
 #else
 typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, /*A K-major*/ true, /*B K-major*/ false, RD_VEC != 0> CfgNN;
 typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, true, true, RD_VEC != 0> CfgNT;
