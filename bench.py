@@ -157,8 +157,8 @@ def main():
                     "unit": "TFLOP/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["traffic"] = None
-    roof["kernel"] = {"fwd": "gmm_kernel (NN)" if name != "decode" else "gmm_decode_kernel", "dlhs": "gmm_kernel (NT)",
-                      "drhs": "tgmm_kernel"}[dominant]
+    roof["kernel"] = {"fwd": "gmm_kernel<.., trans_rhs=false>" if name != "decode" else "gmm_decode_kernel",
+                      "dlhs": "gmm_kernel<.., trans_rhs=true>", "drhs": "tgmm_kernel"}[dominant]
     roof["launch_ms"] = per[dominant]
 
     plans = {}

@@ -50,10 +50,15 @@ class VariantInfo(ctypes.Structure):
 
 
 class Plan(ctypes.Structure):
-    _fields_ = [("variant", ctypes.c_int), ("group_m", ctypes.c_int), ("decode_nb", ctypes.c_int)]
+    _fields_ = [("variant", ctypes.c_int), ("group_m", ctypes.c_int), ("group_n", ctypes.c_int),
+                ("decode_nb", ctypes.c_int)]
+
+    def __init__(self, variant=-1, group_m=0, decode_nb=0, group_n=0):
+        super().__init__(variant, group_m, group_n, decode_nb)
 
     def __repr__(self):
-        return f"Plan(variant={self.variant}, group_m={self.group_m}, decode_nb={self.decode_nb})"
+        return (f"Plan(variant={self.variant}, group_m={self.group_m}, group_n={self.group_n}, "
+                f"decode_nb={self.decode_nb})")
 
 
 # every symbol the header declares; checked at load time

@@ -31,6 +31,10 @@ struct DldsCfg {
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   static constexpr int TM = WM / 32, TN = WN / 32;
   static constexpr int KSTEPS = BK / 16;
+  // Tiles whose accumulators take <= 64 registers leave room for a second (third) work-group on the CU, which hides
+  // the fill and drain of short K loops; tell the register allocator so.
+  static constexpr int TARGET_WGS = (TM * TN * 16 <= 64) ? (NW >= 8 ? 2 : 3) : 1;
+  static constexpr int WAVES_PER_EU = (NW / 4) * TARGET_WGS;
   static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
   // The epilogue re-uses LDS to turn accumulators into row-contiguous 16-byte stores: one [WM][WN] bf16 patch per
@@ -43,7 +47,7 @@ struct DldsCfg {
   static_assert(BM % 128 == 0 && BN % 128 == 0, "direct-to-LDS tiles are at least 128 wide");
   static_assert(BM % (32 * WAVES_M) == 0 && BN % (32 * WAVES_N) == 0, "tile shape");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
-  static_assert(!PINGPONG || (NW == 8 && WAVES_M == 2 && STAGES >= 2), "ping-pong runs two groups of four waves");
+  static_assert(!PINGPONG || (NW == 8 && WAVES_M == 2 && STAGES >= 3), "ping-pong runs two groups of four waves");
 };
 
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
@@ -92,11 +96,11 @@ struct DldsLoader {
       const int pchunk = lane % CPR;
       if (KMAJOR) {
         const int c = pchunk ^ (BK == 64 ? ((r >> 1) & 7) : ((r >> 2) & 3));
-        voff[j] = (imin(r, lim - 1) * ld + c * 8) * 2;
+        voff[j] = r < lim ? (r * ld + c * 8) * 2 : kOobOffset;  // rows past the tile's limit: no memory access, zeros
         kcol = c * 8;  // identical for every j: r advances by a multiple of 16 rows per instruction slot
       } else {
         const int c = pchunk ^ ((r & 3) << 2);
-        voff[j] = (r * ld + imin(c * 8, lim - 8)) * 2;
+        voff[j] = c * 8 < lim ? (r * ld + c * 8) * 2 : kOobOffset;
       }
     }
   }
@@ -218,6 +222,9 @@ __device__ __forceinline__ void gemm_tile_dlds(const bf16_bits* __restrict__ Ap,
   DldsFragReader<C::BN, C::BK, C::TN, C::B_KMAJOR> frb;
   fra.init(wm * C::WM, lane);
   frb.init(wn * C::WN, lane);
+  // A group's last tile (and most tiles of a short group) has few valid rows: a wave whose whole patch lies past the
+  // tile's limits skips its matrix-core work.
+  const bool patch_live = wm * C::WM < a_lim && wn * C::WN < b_lim;
 
   f32x16_t acc[C::TM][C::TN];
 #pragma unroll
@@ -290,11 +297,13 @@ __device__ __forceinline__ void gemm_tile_dlds(const bf16_bits* __restrict__ Ap,
       }
       // Keep the compiler from sinking those reads and loads below the matrix-core work they are meant to overlap.
       __builtin_amdgcn_sched_barrier(0);
+      if (patch_live) {
 #pragma unroll
-      for (int i = 0; i < C::TM; ++i)
+        for (int i = 0; i < C::TM; ++i)
 #pragma unroll
-        for (int j = 0; j < C::TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
+          for (int j = 0; j < C::TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
     if (more) { la.advance(); lb.advance(); }
@@ -329,6 +338,9 @@ __device__ __forceinline__ void gemm_tile_pingpong(const bf16_bits* __restrict__
   DldsFragReader<C::BN, C::BK, C::TN, C::B_KMAJOR> frb;
   fra.init(wm * C::WM, lane);
   frb.init(wn * C::WN, lane);
+  // A group's last tile (and most tiles of a short group) has few valid rows: a wave whose whole patch lies past the
+  // tile's limits skips its matrix-core work.
+  const bool patch_live = wm * C::WM < a_lim && wn * C::WN < b_lim;
 
   f32x16_t acc[C::TM][C::TN];
 #pragma unroll
@@ -391,116 +403,16 @@ __device__ __forceinline__ void gemm_tile_pingpong(const bf16_bits* __restrict__
     __builtin_amdgcn_sched_barrier(0);
     // ---- compute phase ------------------------------------------------------------------------------------------
     __builtin_amdgcn_s_setprio(1);
+    if (patch_live) {
 #pragma unroll
-    for (int ks = 0; ks < C::KSTEPS; ++ks)
+      for (int ks = 0; ks < C::KSTEPS; ++ks)
 #pragma unroll
-      for (int i = 0; i < C::TM; ++i)
+        for (int i = 0; i < C::TM; ++i)
 #pragma unroll
-        for (int j = 0; j < C::TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
+          for (int j = 0; j < C::TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
+    }
     __builtin_amdgcn_s_setprio(0);
-    __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  if (group == 0) __builtin_amdgcn_s_barrier();
-
-  store_accumulators<C>(acc, wm, wn, wave, lane, a_lim, b_lim, Op, ldo, smem);
-}
-
-// Ping-pong on a two-slot ring (room for 64-wide K-slabs, which keep K-major operands on whole 128-byte lines).
-// With only two slots a slab can be requested no earlier than two phases before its first use, so both groups issue
-// their share of slab kt+1 at the start of the same interval: the first group at the head of its memory phase, the
-// second at the head of its compute phase.
-template <class C>
-__device__ __forceinline__ void gemm_tile_pingpong2(const bf16_bits* __restrict__ Ap, int lda, int a_lim,
-                                                    const bf16_bits* __restrict__ Bp, int ldb, int b_lim, int klen,
-                                                    bf16_bits* __restrict__ Op, int ldo, bf16_bits* smem_) {
-  static_assert(C::STAGES == 2, "two-slot ring");
-  unsigned char* smem = reinterpret_cast<unsigned char*>(smem_);
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;
-  const int group = wave >> 2;
-
-  typedef DldsLoader<C::BM, C::BK, C::NW, C::A_KMAJOR> LdA;
-  typedef DldsLoader<C::BN, C::BK, C::NW, C::B_KMAJOR> LdB;
-  LdA la; LdB lb;
-  la.init(Ap, lda, a_lim, klen, wave, lane);
-  lb.init(Bp, ldb, b_lim, klen, wave, lane);
-  DldsFragReader<C::BM, C::BK, C::TM, C::A_KMAJOR> fra;
-  DldsFragReader<C::BN, C::BK, C::TN, C::B_KMAJOR> frb;
-  fra.init(wm * C::WM, lane);
-  frb.init(wn * C::WN, lane);
-
-  f32x16_t acc[C::TM][C::TN];
-#pragma unroll
-  for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-    for (int j = 0; j < C::TN; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-
-  const int nk = (klen + C::BK - 1) / C::BK;
-
-  auto issue_slab = [&](int step) {
-    unsigned char* st = smem + (step & 1) * C::STAGE_BYTES;
-    const int k0 = step * C::BK;
-    const bool tail = k0 + C::BK > klen;
-    __amdgpu_buffer_rsrc_t ra_ = la.resource(), rb_ = lb.resource();
-#pragma unroll
-    for (int q = 0; q < LdA::PER; ++q) {
-      if (tail) la.template issue<true>(ra_, st, wave, q, k0, klen);
-      else la.template issue<false>(ra_, st, wave, q, k0, klen);
-    }
-#pragma unroll
-    for (int q = 0; q < LdB::PER; ++q) {
-      if (tail) lb.template issue<true>(rb_, st + C::A_BYTES, wave, q, k0, klen);
-      else lb.template issue<false>(rb_, st + C::A_BYTES, wave, q, k0, klen);
-    }
-    la.advance();
-    lb.advance();
-  };
-
-  if (nk > 0) issue_slab(0);
-  wait_vmcnt<0>();
-  __builtin_amdgcn_s_barrier();
-  if (group == 1) {
-    if (1 < nk) issue_slab(1);
-    __builtin_amdgcn_s_barrier();
-  }
-
-  for (int kt = 0; kt < nk; ++kt) {
-    // ---- memory phase -------------------------------------------------------------------------------------------
-    if (group == 0 && kt + 1 < nk) issue_slab(kt + 1);
-    const unsigned char* ra = smem + (kt & 1) * C::STAGE_BYTES;
-    const unsigned char* rb = ra + C::A_BYTES;
-    bf16x8_t fa[C::KSTEPS][C::TM], fb[C::KSTEPS][C::TN];
-#pragma unroll
-    for (int ks = 0; ks < C::KSTEPS; ++ks) {
-#pragma unroll
-      for (int i = 0; i < C::TM; ++i) fa[ks][i] = fra.read(ra, i, ks);
-#pragma unroll
-      for (int j = 0; j < C::TN; ++j) fb[ks][j] = frb.read(rb, j, ks);
-    }
-    if (group == 1) wait_vmcnt<0>();       // second group's share of slab kt+1 (requested during its last compute phase)
-    __builtin_amdgcn_s_waitcnt(0xc07f);    // lgkmcnt(0): fragments are in registers, the slot may be refilled
-    __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-    // ---- compute phase ------------------------------------------------------------------------------------------
-    if (group == 1 && kt + 2 < nk) issue_slab(kt + 2);
-    __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_setprio(1);
-#pragma unroll
-    for (int ks = 0; ks < C::KSTEPS; ++ks)
-#pragma unroll
-      for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-        for (int j = 0; j < C::TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
-    __builtin_amdgcn_s_setprio(0);
-    if (group == 0) wait_vmcnt<0>();       // first group's share of slab kt+1
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);

@@ -26,6 +26,7 @@ struct TileCfg {
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // per-wave tile
   static constexpr int TM = WM / 32, TN = WN / 32;       // 32x32 MFMA tiles per wave
   static constexpr int KSTEPS = BK / 16;
+  static constexpr int WAVES_PER_EU = NT >= 256 ? NT / 256 : 1;
   // LDS row pitches (elements).  K-major rows get 16 B of padding: 16 consecutive rows then start in 16 different
   // 16-byte bank groups.  MN-major rows get 64 B: the 4 rows touched by one transposing read land in different
   // quarters of the 256-byte bank window.

@@ -19,7 +19,7 @@ struct GmmArgs {
   int m, k, n, g;
   int U;        // static bound on row tiles: ceil(m / BM) + g
   int n_tiles;  // ceil(n / BN)
-  int group_m;  // row tiles per band of the tile walk
+  int group_m, group_n;  // tiles per L2-sharing block of the tile walk (rows x columns)
 };
 
 // dA[g, k, n] = x[rows of g, k]^T . dy[rows of g, n]
@@ -40,8 +40,7 @@ __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirs
 template <class C>
 __device__ __forceinline__ void run_tile(const bf16_bits* Ap, int lda, int a_lim, const bf16_bits* Bp, int ldb,
                                          int b_lim, int klen, bf16_bits* Op, int ldo, bf16_bits* smem) {
-  if constexpr (C::DLDS && C::PINGPONG && C::STAGES == 2) gemm_tile_pingpong2<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
-  else if constexpr (C::DLDS && C::PINGPONG) gemm_tile_pingpong<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
+  if constexpr (C::DLDS && C::PINGPONG) gemm_tile_pingpong<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
   else if constexpr (C::DLDS) gemm_tile_dlds<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
   else gemm_tile<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
 }
@@ -58,12 +57,20 @@ __device__ __forceinline__ void band_walk(int id, int rows, int cols, int group_
 }
 
 template <class C, bool TRANS_RHS>
-__global__ __launch_bounds__(C::NT) void gmm_kernel(GmmArgs p) {
+__global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) {
   extern __shared__ __attribute__((aligned(16))) bf16_bits smem[];
-  const int id = xcd_contiguous_id(blockIdx.x, p.U * p.n_tiles);
-  if (id < 0) return;
-  int mi, nj;
-  band_walk(id, p.U, p.n_tiles, p.group_m, mi, nj);
+  // Tile walk.  Tiles are grouped into blocks of group_m x group_n (about as many as one XCD runs at a time, so the
+  // block's operand slabs are fetched into that XCD's L2 once), and blocks are dealt to the 8 XCDs (launch index mod 8)
+  // round-robin.  Consecutive row tiles therefore spread over all XCDs, which keeps them evenly loaded when a few
+  // groups are much longer than the rest and their tiles cost more than the mostly-empty ones.
+  const int per_block = p.group_m * p.group_n;
+  const int block_cols = (p.n_tiles + p.group_n - 1) / p.group_n;
+  const int pos = blockIdx.x >> 3;
+  const int block = (pos / per_block) * 8 + (blockIdx.x & 7);
+  const int q = pos % per_block;
+  const int mi = (block / block_cols) * p.group_m + q % p.group_m;
+  const int nj = (block % block_cols) * p.group_n + q / p.group_m;
+  if (mi >= p.U || nj >= p.n_tiles) return;
 
   // Everything read through the map is the same for the whole work-group: pin it to scalar registers.
   const int total = imin(uniform(*p.total_tiles), p.U);
@@ -95,14 +102,20 @@ __global__ __launch_bounds__(C::NT) void gmm_kernel(GmmArgs p) {
 }
 
 template <class C>
-__global__ __launch_bounds__(C::NT) void tgmm_kernel(TgmmArgs p) {
+__global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void tgmm_kernel(TgmmArgs p) {
   extern __shared__ __attribute__((aligned(16))) bf16_bits smem[];
+  // Work per tile is proportional to its group's row count, which only the device knows and which can be wildly
+  // skewed.  So every XCD (launch index mod 8) takes one eighth of every group's tiles - a contiguous stretch of the
+  // group's banded walk, so its tiles still share operand columns in its L2 - and all XCDs get the same share of every
+  // group however the rows are distributed.
   const int per_group = p.k_tiles * p.n_tiles;
-  const int id = xcd_contiguous_id(blockIdx.x, p.g * per_group);
-  if (id < 0) return;
-  const int gi = id / per_group;
+  const int quota = (per_group + 7) >> 3;  // tiles of one group per XCD
+  const int xcd = blockIdx.x & 7, pos = blockIdx.x >> 3;
+  const int gi = pos / quota;
+  const int t = ((xcd + gi) & 7) * quota + (pos - gi * quota);
+  if (gi >= p.g || t >= per_group) return;
   int ri, cj;
-  band_walk(id - gi * per_group, p.k_tiles, p.n_tiles, p.group_m, ri, cj);
+  band_walk(t, p.k_tiles, p.n_tiles, p.group_m, ri, cj);
 
   const int kk0 = ri * C::BM, col0 = cj * C::BN;
   const int krows = imin(C::BM, p.k - kk0), cols = imin(C::BN, p.n - col0);
@@ -146,7 +159,8 @@ int launch_gmm(hipStream_t s, const GmmArgs& a) {
   auto kern = gmm_kernel<C, TRANS_RHS>;
   const int attr_rc = allow_big_lds(reinterpret_cast<const void*>(kern), C::LDS_BYTES);
   if (attr_rc != hipSuccess) return attr_rc;
-  const int grid = xcd_padded_grid(a.U * a.n_tiles);
+  const int blocks = ((a.U + a.group_m - 1) / a.group_m) * ((a.n_tiles + a.group_n - 1) / a.group_n);
+  const int grid = 8 * ((blocks + 7) / 8) * a.group_m * a.group_n;
   if (grid <= 0) return hipSuccess;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(C::NT), C::LDS_BYTES, s, a);
   return (int)hipGetLastError();
@@ -157,7 +171,7 @@ int launch_tgmm(hipStream_t s, const TgmmArgs& a) {
   auto kern = tgmm_kernel<C>;
   const int attr_rc = allow_big_lds(reinterpret_cast<const void*>(kern), C::LDS_BYTES);
   if (attr_rc != hipSuccess) return attr_rc;
-  const int grid = xcd_padded_grid(a.g * a.k_tiles * a.n_tiles);
+  const int grid = 8 * a.g * ((a.k_tiles * a.n_tiles + 7) / 8);
   if (grid <= 0) return hipSuccess;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(C::NT), C::LDS_BYTES, s, a);
   return (int)hipGetLastError();

@@ -94,7 +94,8 @@ def select_plan(
     vec = k % 8 == 0 and n % 8 == 0
     entry = tuned_plans().get(plan_key(op, m, k, n, g))
     if entry is not None and vec:
-        plan = _capi.Plan(variant_id(entry["variant"]), int(entry.get("group_m", 0)), int(entry.get("decode_nb", 0)))
+        plan = _capi.Plan(variant_id(entry["variant"]), int(entry.get("group_m", 0)), int(entry.get("decode_nb", 0)),
+                          int(entry.get("group_n", 0)))
         return plan
     plan = _capi.default_plan(op, m, k, n, g)
     if (block_m, block_k, block_n) != (DEFAULT_BLOCK_M, DEFAULT_BLOCK_K, DEFAULT_BLOCK_N) and not plan.decode_nb:

@@ -51,7 +51,8 @@ typedef struct rd_variant_info {
 /* Launch plan for one call; the host planner (or the caller) fills it.  Zero-initialised = library defaults. */
 typedef struct rd_plan {
   int variant; /* index into the variant table, or -1: let the library choose by shape */
-  int group_m; /* row tiles per band of the tile walk (L2 reuse); 0 = default */
+  int group_m; /* tile walk: row tiles per L2-sharing block (tgmm: per band); 0 = default */
+  int group_n; /* tile walk: column tiles per block (rd_gmm only); 0 = default */
   int decode_nb; /* rd_gmm only: > 0 selects the skinny-m streaming kernel with this many columns per work-group */
 } rd_plan;
 
