@@ -84,6 +84,8 @@ def main():
     ap.add_argument("--workload", default="mixtral_fwd_bwd")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy, so a counter run has a kernel of known traffic to scale by")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU: the ragged_dot path has no multi-GPU part; run with --gpus 1")
@@ -124,6 +126,14 @@ def main():
         for _, fn in parts:
             fn()
 
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -156,7 +166,12 @@ def main():
             roof = {"bound": "mfma", "achieved": flops_one / (per[dominant] * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
                     "unit": "TFLOP/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = None
+    roof["traffic"] = None  # HBM bytes per launch of the dominant kernel, from committed counter runs (profiles/)
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            roof["traffic"] = json.load(f).get(name, {}).get(dominant)
+    except (OSError, ValueError):
+        pass
     roof["kernel"] = {"fwd": "gmm_kernel<.., trans_rhs=false>" if name != "decode" else "gmm_decode_kernel",
                       "dlhs": "gmm_kernel<.., trans_rhs=true>", "drhs": "tgmm_kernel"}[dominant]
     roof["launch_ms"] = per[dominant]
