@@ -92,13 +92,13 @@ def select_plan(
 ) -> _capi.Plan:
     """Plan for op (0 gmm, 1 gmm with trans_rhs, 2 tgmm) on a bf16 problem of this shape."""
     vec = k % 8 == 0 and n % 8 == 0
+    explicit = (block_m, block_k, block_n) != (DEFAULT_BLOCK_M, DEFAULT_BLOCK_K, DEFAULT_BLOCK_N)
     entry = tuned_plans().get(plan_key(op, m, k, n, g))
-    if entry is not None and vec:
-        plan = _capi.Plan(variant_id(entry["variant"]), int(entry.get("group_m", 0)), int(entry.get("decode_nb", 0)),
+    if entry is not None and vec and not explicit:
+        return _capi.Plan(variant_id(entry["variant"]), int(entry.get("group_m", 0)), int(entry.get("decode_nb", 0)),
                           int(entry.get("group_n", 0)))
-        return plan
     plan = _capi.default_plan(op, m, k, n, g)
-    if (block_m, block_k, block_n) != (DEFAULT_BLOCK_M, DEFAULT_BLOCK_K, DEFAULT_BLOCK_N) and not plan.decode_nb:
+    if explicit and not plan.decode_nb:
         # explicit request: nearest compiled shape.  For tgmm the output tile is (block_k, block_n).
         want_rows = block_k if op == _capi.OP_TGMM else block_m
         best, best_d = None, None
