@@ -2,6 +2,7 @@
 // map, tail / empty-group zeroing.
 #pragma once
 #include "rd_gemm_dlds.h"
+#include "rd_gemm_pp.h"
 #include "rd_gemm_tile.h"
 
 namespace rd {
@@ -40,7 +41,8 @@ __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirs
 template <class C>
 __device__ __forceinline__ void run_tile(const bf16_bits* Ap, int lda, int a_lim, const bf16_bits* Bp, int ldb,
                                          int b_lim, int klen, bf16_bits* Op, int ldo, bf16_bits* smem) {
-  if constexpr (C::DLDS && C::PINGPONG) gemm_tile_pingpong<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
+  if constexpr (C::MIXED) gemm_tile_pingpong_mixed<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
+  else if constexpr (C::DLDS && C::PINGPONG) gemm_tile_pingpong<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
   else if constexpr (C::DLDS) gemm_tile_dlds<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
   else gemm_tile<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
 }

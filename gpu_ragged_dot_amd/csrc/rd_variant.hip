@@ -1,5 +1,5 @@
 // One compiled tile shape.  Built once per entry of the variant list in the Makefile, with
-//   -DRD_BM= -DRD_BN= -DRD_BK= -DRD_WAVES_M= -DRD_WAVES_N= -DRD_VEC= -DRD_NAME= [-DRD_DLDS=1 -DRD_STAGES= -DRD_PINGPONG=1]
+//   -DRD_BM= -DRD_BN= -DRD_BK= -DRD_WAVES_M= -DRD_WAVES_N= -DRD_VEC= -DRD_NAME= [-DRD_DLDS=1|2 -DRD_STAGES= -DRD_PINGPONG=1]
 // and exports a getter rd_variant_<name>() for its TileVariant record that the C-ABI file collects.
 #include "rd_kernels.h"
 
@@ -19,7 +19,12 @@
 #endif
 
 namespace rd {
-#if RD_DLDS
+#if RD_DLDS == 2
+// one LDS ring per operand: K-major A in 64-wide slabs (3 slots), everything else in 32-wide slabs (4 slots)
+typedef PpCfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, /*A K-major*/ true, /*B K-major*/ false, 64, 3, 32, 4> CfgNN;
+typedef PpCfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, true, true, 64, 3, 32, 4> CfgNT;
+typedef PpCfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, false, false, 32, 4, 32, 4> CfgTN;
+#elif RD_DLDS
 typedef DldsCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, /*A K-major*/ true, /*B K-major*/ false, RD_STAGES, RD_PINGPONG != 0> CfgNN;
 typedef DldsCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, true, true, RD_STAGES, RD_PINGPONG != 0> CfgNT;
 typedef DldsCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, false, false, RD_STAGES, RD_PINGPONG != 0> CfgTN;
@@ -32,7 +37,7 @@ typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, false, false, RD_VE
 
 extern "C" const rd::TileVariant* RD_CAT(rd_variant_, RD_NAME)() {
   static const rd::TileVariant v = {
-      RD_STR(RD_NAME), RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, RD_VEC, RD_DLDS, RD_STAGES,
+      RD_STR(RD_NAME), RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, RD_VEC, RD_DLDS != 0, RD_STAGES,
       &rd::launch_gmm<rd::CfgNN, false>, &rd::launch_gmm<rd::CfgNT, true>, &rd::launch_tgmm<rd::CfgTN>};
   return &v;
 }
