@@ -43,6 +43,7 @@ class VariantInfo(ctypes.Structure):
         ("waves_m", ctypes.c_int),
         ("waves_n", ctypes.c_int),
         ("vec", ctypes.c_int),
+        ("dtype", ctypes.c_int),
         ("direct_to_lds", ctypes.c_int),
         ("stages", ctypes.c_int),
         ("name", ctypes.c_char * 48),

@@ -24,6 +24,8 @@ namespace rd {
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, bool A_KMAJOR_, bool B_KMAJOR_, int STAGES_,
           bool PINGPONG_ = false>
 struct DldsCfg {
+  typedef bf16_bits Elem;
+  static constexpr bool F32 = false;
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
   static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = true, DLDS = true, PINGPONG = PINGPONG_, MIXED = false;
   static constexpr int NW = WAVES_M * WAVES_N;

@@ -11,6 +11,8 @@ namespace rd {
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, bool A_KMAJOR_, bool B_KMAJOR_, int A_W_, int A_S_, int B_W_,
           int B_S_>
 struct PpCfg {
+  typedef bf16_bits Elem;
+  static constexpr bool F32 = false;
   static constexpr int BM = BM_, BN = BN_, BK = 32, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
   static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = true, DLDS = true, PINGPONG = true, MIXED = true;
   static constexpr int A_W = A_W_, A_S = A_S_, B_W = B_W_, B_S = B_S_;  // slab width (contraction), ring slots

@@ -19,6 +19,8 @@ namespace rd {
 
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, bool A_KMAJOR_, bool B_KMAJOR_, bool VEC_>
 struct TileCfg {
+  typedef bf16_bits Elem;
+  static constexpr bool F32 = false;
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
   static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = VEC_, DLDS = false, PINGPONG = false, MIXED = false;
   static constexpr int STAGES = 2;
@@ -208,9 +210,9 @@ __device__ __forceinline__ void gemm_tile(const bf16_bits* __restrict__ Ap, int 
 }
 
 // Zero rows [0, rows) x cols [0, cols) of a bf16 matrix with pitch ld, all threads of the work-group cooperating.
-template <int NT, bool VEC>
-__device__ __forceinline__ void zero_tile(bf16_bits* __restrict__ Op, int ld, int rows, int cols) {
-  if (VEC) {  // cols % 8 == 0 and 16-byte aligned rows
+template <int NT, bool VEC, typename E>
+__device__ __forceinline__ void zero_tile(E* __restrict__ Op, int ld, int rows, int cols) {
+  if (VEC && sizeof(E) == 2) {  // cols % 8 == 0 and 16-byte aligned rows
     const int cpr = cols >> 3;
     for (int idx = threadIdx.x; idx < rows * cpr; idx += NT) {
       const int r = idx / cpr, c = idx - r * cpr;

@@ -2,6 +2,7 @@
 // map, tail / empty-group zeroing.
 #pragma once
 #include "rd_gemm_dlds.h"
+#include "rd_gemm_f32.h"
 #include "rd_gemm_pp.h"
 #include "rd_gemm_tile.h"
 
@@ -9,9 +10,9 @@ namespace rd {
 
 // y[m, n] = ragged x[m, k] . A[g]  (A is [g, k, n], or [g, n, k] when trans_rhs).
 struct GmmArgs {
-  const bf16_bits* x;
-  const bf16_bits* A;
-  bf16_bits* y;
+  const void* x;  // element type is the kernel configuration's Elem (bf16 bits or float)
+  const void* A;
+  void* y;
   const int32_t* group_sizes;    // [g]
   const int32_t* group_offsets;  // [g]   exclusive prefix sum of group_sizes
   const int32_t* tile2group;     // [U]   scheduling map built with chunk = tile height
@@ -25,9 +26,9 @@ struct GmmArgs {
 
 // dA[g, k, n] = x[rows of g, k]^T . dy[rows of g, n]
 struct TgmmArgs {
-  const bf16_bits* x;
-  const bf16_bits* dy;
-  bf16_bits* dA;
+  const void* x;
+  const void* dy;
+  void* dA;
   const int32_t* group_sizes;
   const int32_t* group_offsets;
   int m, k, n, g;
@@ -39,9 +40,11 @@ struct TgmmArgs {
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
 template <class C>
-__device__ __forceinline__ void run_tile(const bf16_bits* Ap, int lda, int a_lim, const bf16_bits* Bp, int ldb,
-                                         int b_lim, int klen, bf16_bits* Op, int ldo, bf16_bits* smem) {
-  if constexpr (C::MIXED) gemm_tile_pingpong_mixed<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
+__device__ __forceinline__ void run_tile(const typename C::Elem* Ap, int lda, int a_lim, const typename C::Elem* Bp,
+                                         int ldb, int b_lim, int klen, typename C::Elem* Op, int ldo,
+                                         typename C::Elem* smem) {
+  if constexpr (C::F32) gemm_tile_f32<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
+  else if constexpr (C::MIXED) gemm_tile_pingpong_mixed<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
   else if constexpr (C::DLDS && C::PINGPONG) gemm_tile_pingpong<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
   else if constexpr (C::DLDS) gemm_tile_dlds<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
   else gemm_tile<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
@@ -60,7 +63,12 @@ __device__ __forceinline__ void band_walk(int id, int rows, int cols, int group_
 
 template <class C, bool TRANS_RHS>
 __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) {
-  extern __shared__ __attribute__((aligned(16))) bf16_bits smem[];
+  typedef typename C::Elem E;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  E* smem = reinterpret_cast<E*>(smem_raw);
+  const E* px = static_cast<const E*>(p.x);
+  const E* pA = static_cast<const E*>(p.A);
+  E* py = static_cast<E*>(p.y);
   // Tile walk.  Tiles are grouped into blocks of group_m x group_n (about as many as one XCD runs at a time, so the
   // block's operand slabs are fetched into that XCD's L2 once), and blocks are dealt to the 8 XCDs (launch index mod 8)
   // round-robin.  Consecutive row tiles therefore spread over all XCDs, which keeps them evenly loaded when a few
@@ -86,10 +94,9 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
     int rows = imin(C::BM, uniform(p.group_sizes[gi]) - it * C::BM);
     rows = imin(rows, p.m - row0);  // group_sizes summing past m: never touch rows >= m
     if (rows <= 0 || row0 < 0) return;
-    const bf16_bits* Ap = p.x + (size_t)row0 * p.k;
-    const bf16_bits* Bp = TRANS_RHS ? p.A + (size_t)gi * p.n * p.k + (size_t)col0 * p.k
-                                    : p.A + (size_t)gi * p.k * p.n + col0;
-    bf16_bits* Op = p.y + (size_t)row0 * p.n + col0;
+    const E* Ap = px + (size_t)row0 * p.k;
+    const E* Bp = TRANS_RHS ? pA + (size_t)gi * p.n * p.k + (size_t)col0 * p.k : pA + (size_t)gi * p.k * p.n + col0;
+    E* Op = py + (size_t)row0 * p.n + col0;
     run_tile<C>(Ap, p.k, rows, Bp, TRANS_RHS ? p.k : p.n, cols, p.k, Op, p.n, smem);
   } else {
     // Rows past sum(group_sizes) are defined to be zero.  The map never uses more than
@@ -99,13 +106,15 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
     const long long r0 = s + (long long)(mi - total) * C::BM;
     if (r0 >= p.m) return;
     const int rows = imin(C::BM, p.m - (int)r0);
-    zero_tile<C::NT, C::VEC>(p.y + (size_t)r0 * p.n + col0, p.n, rows, cols);
+    zero_tile<C::NT, C::VEC, E>(py + (size_t)r0 * p.n + col0, p.n, rows, cols);
   }
 }
 
 template <class C>
 __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void tgmm_kernel(TgmmArgs p) {
-  extern __shared__ __attribute__((aligned(16))) bf16_bits smem[];
+  typedef typename C::Elem E;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  E* smem = reinterpret_cast<E*>(smem_raw);
   // Work per tile is proportional to its group's row count, which only the device knows and which can be wildly
   // skewed.  So every XCD (launch index mod 8) takes one eighth of every group's tiles - a contiguous stretch of the
   // group's banded walk, so its tiles still share operand columns in its L2 - and all XCDs get the same share of every
@@ -121,17 +130,17 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void tgmm_kernel(TgmmArgs p
 
   const int kk0 = ri * C::BM, col0 = cj * C::BN;
   const int krows = imin(C::BM, p.k - kk0), cols = imin(C::BN, p.n - col0);
-  bf16_bits* Op = p.dA + (size_t)gi * p.k * p.n + (size_t)kk0 * p.n + col0;
+  E* Op = static_cast<E*>(p.dA) + (size_t)gi * p.k * p.n + (size_t)kk0 * p.n + col0;
 
   const int row0 = uniform(p.group_offsets[gi]);
   int rows = uniform(p.group_sizes[gi]);
   rows = imin(rows, p.m - row0);
   if (rows <= 0 || row0 < 0) {  // empty group: its slice of dA is zero
-    zero_tile<C::NT, C::VEC>(Op, p.n, krows, cols);
+    zero_tile<C::NT, C::VEC, E>(Op, p.n, krows, cols);
     return;
   }
-  const bf16_bits* Ap = p.x + (size_t)row0 * p.k + kk0;
-  const bf16_bits* Bp = p.dy + (size_t)row0 * p.n + col0;
+  const E* Ap = static_cast<const E*>(p.x) + (size_t)row0 * p.k + kk0;
+  const E* Bp = static_cast<const E*>(p.dy) + (size_t)row0 * p.n + col0;
   run_tile<C>(Ap, p.k, krows, Bp, p.n, cols, rows, Op, p.n, smem);
 }
 
@@ -144,6 +153,7 @@ struct TileVariant {
   const char* name;
   int bm, bn, bk, waves_m, waves_n;
   int vec;  // 1: needs k % 8 == 0 and n % 8 == 0 (16-byte row pitches); 0: any shape
+  int f32;     // 1: float32 operands and output; 0: bf16
   int dlds;    // 1: direct-to-LDS core (byte extents of one tile's operand window must stay below 2 GiB)
   int stages;  // LDS ring depth
   gmm_launch_fn gmm_nn, gmm_nt;

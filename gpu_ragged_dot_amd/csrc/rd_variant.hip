@@ -18,8 +18,16 @@
 #define RD_PINGPONG 0
 #endif
 
+#ifndef RD_F32
+#define RD_F32 0
+#endif
+
 namespace rd {
-#if RD_DLDS == 2
+#if RD_F32
+typedef F32Cfg</*A K-major*/ true, /*B K-major*/ false> CfgNN;
+typedef F32Cfg<true, true> CfgNT;
+typedef F32Cfg<false, false> CfgTN;
+#elif RD_DLDS == 2
 // one LDS ring per operand: K-major A in 64-wide slabs (3 slots), everything else in 32-wide slabs (4 slots)
 typedef PpCfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, /*A K-major*/ true, /*B K-major*/ false, 64, 3, 32, 4> CfgNN;
 typedef PpCfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, true, true, 64, 3, 32, 4> CfgNT;
@@ -37,7 +45,7 @@ typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, false, false, RD_VE
 
 extern "C" const rd::TileVariant* RD_CAT(rd_variant_, RD_NAME)() {
   static const rd::TileVariant v = {
-      RD_STR(RD_NAME), RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, RD_VEC, RD_DLDS != 0, RD_STAGES,
+      RD_STR(RD_NAME), RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, RD_VEC, RD_F32, RD_DLDS != 0, RD_STAGES,
       &rd::launch_gmm<rd::CfgNN, false>, &rd::launch_gmm<rd::CfgNT, true>, &rd::launch_tgmm<rd::CfgTN>};
   return &v;
 }

@@ -22,7 +22,7 @@ _DTYPES = {torch.bfloat16: _capi.RD_DTYPE_BF16, torch.float32: _capi.RD_DTYPE_F3
 
 def _dtype_code(t: torch.Tensor, compute_dtype, acc_dtype) -> int:
     if t.dtype not in _DTYPES:
-        raise TypeError(f"unsupported dtype {t.dtype}; bf16 is the compiled operand type")
+        raise TypeError(f"unsupported dtype {t.dtype}; operands are bfloat16 or float32")
     if compute_dtype is not None and compute_dtype != t.dtype:
         raise NotImplementedError(f"compute_dtype={compute_dtype} differs from the operand dtype {t.dtype}")
     if acc_dtype not in (None, torch.float32):
@@ -81,7 +81,8 @@ def _gmm_fwd(x, A, group_sizes, block_m, block_k, block_n, trans_rhs, interpret,
     gs = _group_sizes_i32(group_sizes, dev)
     y = torch.empty((m, n), dtype=x.dtype, device=dev)  # :210
     if plan is None:
-        plan = planner.select_plan(_capi.OP_GMM_TRANS if trans_rhs else _capi.OP_GMM, m, k, n, g, block_m, block_k, block_n)
+        plan = planner.select_plan(_capi.OP_GMM_TRANS if trans_rhs else _capi.OP_GMM, m, k, n, g, block_m, block_k, block_n,
+                                   dtype=code)
     ws_bytes = _capi.lib.rd_gmm_workspace_bytes(m, g, _plan_ref(plan))
     ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
@@ -111,7 +112,7 @@ def _tgmm_fwd(x, y, group_sizes, block_m, block_k, block_n, interpret, compute_d
     gs = _group_sizes_i32(gs_t, dev)
     out = torch.empty((g, k, n), dtype=x.dtype, device=dev)  # :324
     if plan is None:
-        plan = planner.select_plan(_capi.OP_TGMM, m, k, n, g, block_m, block_k, block_n)
+        plan = planner.select_plan(_capi.OP_TGMM, m, k, n, g, block_m, block_k, block_n, dtype=code)
     ws_bytes = _capi.lib.rd_tgmm_workspace_bytes(m, g, _plan_ref(plan))
     ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):

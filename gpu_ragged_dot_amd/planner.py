@@ -89,8 +89,11 @@ def select_plan(
     block_m: int = DEFAULT_BLOCK_M,
     block_k: int = DEFAULT_BLOCK_K,
     block_n: int = DEFAULT_BLOCK_N,
+    dtype: int = _capi.RD_DTYPE_BF16,
 ) -> _capi.Plan:
-    """Plan for op (0 gmm, 1 gmm with trans_rhs, 2 tgmm) on a bf16 problem of this shape."""
+    """Plan for op (0 gmm, 1 gmm with trans_rhs, 2 tgmm) on a problem of this shape and element type."""
+    if dtype != _capi.RD_DTYPE_BF16:
+        return _capi.default_plan(op, m, k, n, g, dtype)  # one float32 kernel: nothing to choose
     vec = k % 8 == 0 and n % 8 == 0
     explicit = (block_m, block_k, block_n) != (DEFAULT_BLOCK_M, DEFAULT_BLOCK_K, DEFAULT_BLOCK_N)
     entry = tuned_plans().get(plan_key(op, m, k, n, g))
@@ -103,7 +106,7 @@ def select_plan(
         want_rows = block_k if op == _capi.OP_TGMM else block_m
         best, best_d = None, None
         for v in compiled_variants():
-            if bool(v.vec) != vec:
+            if bool(v.vec) != vec or v.dtype != _capi.RD_DTYPE_BF16:
                 continue
             d = abs(math.log2(v.tile_m / max(want_rows, 1))) + abs(math.log2(v.tile_n / max(block_n, 1)))
             if best_d is None or d < best_d:

@@ -52,7 +52,7 @@ def sweep(x, A, dout, gs, op: int, reps: int = 10, rounds: int = 3):
     walks = [(0, 0), (2, 4), (4, 4), (8, 4), (2, 8), (4, 8)] if op != _capi.OP_TGMM else [(4, 0), (8, 0), (16, 0)]
     cands = []
     for v in planner.compiled_variants():
-        if bool(v.vec) != vec:
+        if bool(v.vec) != vec or v.dtype != _capi.RD_DTYPE_BF16:
             continue
         if min(m, 1 << 30) < v.tile_m // 4 and v.tile_m > 64:
             continue

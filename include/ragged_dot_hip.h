@@ -43,6 +43,7 @@ typedef struct rd_variant_info {
   int tile_m, tile_n, tile_k; /* macro-tile: rows x columns x contraction slab */
   int waves_m, waves_n;       /* wavefront grid inside a work-group (64 lanes each) */
   int vec;                    /* 1: needs 16-byte row pitches (k % 8 == 0 and n % 8 == 0 for bf16) */
+  int dtype;                  /* RD_DTYPE_* of operands and output this variant is compiled for */
   int direct_to_lds;          /* 1: HBM -> LDS loads bypass registers; max(m,k)*max(k,n) must stay below 2^30 */
   int stages;                 /* depth of the K-slab ring in LDS */
   char name[48];

@@ -118,7 +118,7 @@ def test_trans_ragged_dot_grid(c):
 # ---------------------------------------------------------------------------------------------------------------------
 
 def _variant_ids():
-    return [(v.id, v.name.decode(), v.vec) for v in _capi.variants()]
+    return [(v.id, v.name.decode(), v.vec) for v in _capi.variants() if v.dtype == _capi.RD_DTYPE_BF16]
 
 
 @pytest.mark.parametrize("vid,vname,vec", _variant_ids(), ids=[v[1] for v in _variant_ids()])
@@ -255,3 +255,57 @@ def test_linearity_and_group_locality():
     same[off[3]:off[4]] = False
     assert torch.equal(y3[same.cuda()], y1[same.cuda()])
     assert torch.equal(y3[off[3]:off[4]].float(), -y1[off[3]:off[4]].float())
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# float32 operands (tests.py:93 runs every test for bfloat16 and float32; eps 5e-4, tgmm 1e-4)
+# ---------------------------------------------------------------------------------------------------------------------
+
+F32_EPS, F32_TGMM_EPS = 5e-4, 1e-4
+
+
+def _f32_case(c):
+    rng = np.random.default_rng(c["seed"] * 101 + c["m"] + c["k"] + c["n"])
+    m, k, n, g = c["m"], c["k"], c["n"], c["g"]
+    if c["random_inputs"]:
+        lhs, rhs, dout = (rng.normal(size=s).astype(np.float32) for s in ((m, k), (g, k, n), (m, n)))
+    else:
+        lhs, rhs, dout = (np.ones(s, np.float32) for s in ((m, k), (g, k, n), (m, n)))
+    target_m = max(min(round(m * c["fill_in"]), m), 0)
+    gs = oracle.generate_group_sizes(c["seed"] + 7 * g + target_m, g, target_m)
+    return lhs, rhs, dout, gs, target_m
+
+
+@pytest.mark.parametrize("trans_rhs", [False, True], ids=["A", "At"])
+@pytest.mark.parametrize("c", GRID[:16], ids=[util.case_id(c) for c in GRID[:16]])
+def test_float32_forward_and_vjp(c, trans_rhs):
+    print("f32", c, "trans_rhs", trans_rhs, flush=True)
+    lhs, rhs, dout, gs, target_m = _f32_case(c)
+    rhs_in = np.ascontiguousarray(np.swapaxes(rhs, 1, 2)) if trans_rhs else rhs
+    x_t = torch.from_numpy(lhs).cuda().requires_grad_(True)
+    A_t = torch.from_numpy(rhs_in).cuda().requires_grad_(True)
+    o = rd.gmm(x_t, A_t, torch.from_numpy(gs), block_m=c["block_m"], block_k=c["block_k"], block_n=c["block_n"],
+               chunk_m=c["chunk_m"], trans_rhs=trans_rhs)
+    assert o.dtype == torch.float32
+    dlhs, drhs = torch.autograd.grad(o, (x_t, A_t), torch.from_numpy(dout).cuda())
+    f64 = dict(out_dtype="float32", acc=np.float64)
+    o_ref = oracle.gmm(lhs, rhs_in, gs, trans_rhs=trans_rhs, **f64)
+    dlhs_ref, drhs_ref, _ = oracle.gmm_vjp(lhs, rhs_in, gs, dout, trans_rhs=trans_rhs, **f64)
+    rows = np.arange(c["m"]) < target_m
+    assert float(np.max(oracle.err_fn(util.to_np(o), o_ref, mask=rows))) < F32_EPS
+    assert float(np.max(oracle.err_fn(util.to_np(dlhs), dlhs_ref, mask=rows))) < F32_EPS
+    assert float(np.max(oracle.err_fn(util.to_np(drhs), drhs_ref, axis=(-1, -2), mask=gs != 0))) < F32_EPS
+    assert not np.any(util.to_np(o)[target_m:]) and not np.any(util.to_np(dlhs)[target_m:])
+    assert not np.any(util.to_np(drhs)[gs == 0])
+    if not c["random_inputs"]:
+        assert np.all(util.to_np(o)[:target_m] == c["k"])
+
+
+@pytest.mark.parametrize("c", GRID[:16], ids=[util.case_id(c) for c in GRID[:16]])
+def test_float32_trans_ragged_dot(c):
+    print("f32 tgmm", c, flush=True)
+    lhs, _, dout, gs, _ = _f32_case(c)
+    out = rd.tgmm(torch.from_numpy(lhs).cuda(), torch.from_numpy(dout).cuda(), torch.from_numpy(gs))
+    ref = oracle.tgmm(lhs, dout, gs, out_dtype="float32", acc=np.float64)
+    assert float(np.max(oracle.err_fn(util.to_np(out), ref, axis=(-1, -2), mask=gs != 0))) < F32_TGMM_EPS
+    assert not np.any(util.to_np(out)[gs == 0])

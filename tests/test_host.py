@@ -35,7 +35,8 @@ def test_variant_table():
     assert len(vs) >= 2
     names = [v.name.decode() for v in vs]
     assert len(set(names)) == len(names)
-    assert any(v.vec == 0 for v in vs), "an any-shape variant must exist for pitches that are not 16-byte multiples"
+    assert any(v.vec == 0 and v.dtype == _capi.RD_DTYPE_BF16 for v in vs), "an any-shape bf16 variant must exist"
+    assert any(v.dtype == _capi.RD_DTYPE_F32 for v in vs), "float32 operands need a kernel too"
     for v in vs:
         assert v.tile_m % (32 * v.waves_m) == 0 and v.tile_n % (32 * v.waves_n) == 0 and v.tile_k % 16 == 0
         if v.direct_to_lds:
@@ -53,7 +54,9 @@ def test_argument_validation_returns_codes():
     assert rc == _capi.RD_ERR_INVALID_ARGUMENT and b"null" in lib.rd_last_error()
     rc = lib.rd_gmm(None, one, one, one, one, 8, 8, 8, 2, 0, 7, None, one, 1 << 20)
     assert rc == _capi.RD_ERR_INVALID_ARGUMENT
-    rc = lib.rd_gmm(None, one, one, one, one, 8, 8, 8, 2, 0, _capi.RD_DTYPE_F32, None, one, 1 << 20)
+    bf16_id = next(v.id for v in _capi.variants() if v.dtype == _capi.RD_DTYPE_BF16 and not v.vec)
+    plan = _capi.Plan(bf16_id, 0, 0)  # a bf16 variant cannot take float32 operands (checked before any launch)
+    rc = lib.rd_gmm(None, one, one, one, one, 8, 8, 8, 2, 0, _capi.RD_DTYPE_F32, ctypes.byref(plan), one, 1 << 20)
     assert rc == _capi.RD_ERR_UNSUPPORTED
     rc = lib.rd_tgmm(None, one, one, one, one, 8, 8, 8, 0, _capi.RD_DTYPE_BF16, None, one, 1 << 20)
     assert rc == _capi.RD_ERR_INVALID_ARGUMENT
@@ -70,7 +73,7 @@ def test_argument_validation_returns_codes():
     assert rc == _capi.RD_ERR_INVALID_ARGUMENT
     rc = lib.rd_gmm(None, one, one, one, one, 64, 64, 64, 2, 0, _capi.RD_DTYPE_BF16, None, one, 8)
     assert rc == _capi.RD_ERR_WORKSPACE
-    vec_id = next(v.id for v in _capi.variants() if v.vec)
+    vec_id = next(v.id for v in _capi.variants() if v.vec and v.dtype == _capi.RD_DTYPE_BF16)
     plan = _capi.Plan(vec_id, 0, 0)
     rc = lib.rd_gmm(None, one, one, one, one, 64, 58, 77, 2, 0, _capi.RD_DTYPE_BF16, ctypes.byref(plan), one, 1 << 20)
     assert rc == _capi.RD_ERR_UNSUPPORTED
@@ -100,6 +103,8 @@ def test_planner_choices():
     vs = {v.id: v for v in _capi.variants()}
     p = planner.select_plan(_capi.OP_GMM, 171, 58, 77, 8)
     assert vs[p.variant].vec == 0 and p.decode_nb == 0  # odd pitches -> any-shape variant
+    p = planner.select_plan(_capi.OP_TGMM, 171, 58, 77, 8, dtype=_capi.RD_DTYPE_F32)
+    assert vs[p.variant].dtype == _capi.RD_DTYPE_F32
     p = planner.select_plan(_capi.OP_GMM, 64, 2048, 768, 128)
     assert p.decode_nb > 0  # a few rows per expert -> streaming kernel
     p = planner.select_plan(_capi.OP_GMM_TRANS, 64, 2048, 768, 128)
