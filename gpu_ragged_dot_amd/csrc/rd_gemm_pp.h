@@ -78,6 +78,7 @@ __device__ __forceinline__ void gemm_tile_pingpong_mixed(const bf16_bits* __rest
                                                          const bf16_bits* __restrict__ Bp, int ldb, int b_lim,
                                                          int klen, bf16_bits* __restrict__ Op, int ldo,
                                                          bf16_bits* smem_) {
+  RD_MARK_DECL;
   unsigned char* smem = reinterpret_cast<unsigned char*>(smem_);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -155,6 +156,16 @@ __device__ __forceinline__ void gemm_tile_pingpong_mixed(const bf16_bits* __rest
     constexpr int KA = C::A_W == 64 ? 2 * PAR : 0, KB = C::B_W == 64 ? 2 * PAR : 0;  // substep offset inside a 64-wide slab
     // ---- memory phase ---------------------------------------------------------------------------------------------
     bf16x8_t fa[C::KSTEPS][C::TM], fb[C::KSTEPS][C::TN];
+    // `steady`: both rings still have a slab to request at their look-ahead distance.  It can only turn false once,
+    // towards the end of the K loop, so while it holds every earlier phase issued its full complement of loads.
+    const bool steady = qa + C::A_S - 1 < na && qb + C::B_S - 1 < nb;
+    const bool do_a = (C::A_W == 32 || PAR == 0) && qa + C::A_S - 1 < na;
+    const bool do_b = (C::B_W == 32 || PAR == 0) && qb + C::B_S - 1 < nb;
+    // Request the far slab before reading this phase's fragments: the texture path takes the requests at its own
+    // pace while the LDS reads run, instead of after them.
+    if (do_a) issue_a(qa + C::A_S - 1);
+    if (do_b) issue_b(qb + C::B_S - 1);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < C::KSTEPS; ++ks) {
 #pragma unroll
@@ -162,21 +173,14 @@ __device__ __forceinline__ void gemm_tile_pingpong_mixed(const bf16_bits* __rest
 #pragma unroll
       for (int j = 0; j < C::TN; ++j) fb[ks][j] = frb.read(rb, j, ks + KB);
     }
-    // `steady`: both rings still have a slab to request at their look-ahead distance.  It can only turn false once,
-    // towards the end of the K loop, so while it holds every earlier phase issued its full complement of loads.
-    const bool steady = qa + C::A_S - 1 < na && qb + C::B_S - 1 < nb;
-    if (C::A_W == 32 || PAR == 0) {
-      if (qa + C::A_S - 1 < na) issue_a(qa + C::A_S - 1);
-    }
-    if (C::B_W == 32 || PAR == 0) {
-      if (qb + C::B_S - 1 < nb) issue_b(qb + C::B_S - 1);
-    }
     // Own share of everything the next phase reads has landed.  The immediate count is exact in the steady state;
     // near the end, where fewer loads are in flight than it assumes, wait for all of them.
     if (steady) wait_vmcnt<Cnt::allowed(PAR)>(); else wait_vmcnt<0>();
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
     __builtin_amdgcn_sched_barrier(0);
+    RD_MARK(0);
     __builtin_amdgcn_s_barrier();
+    RD_MARK(1);
     __builtin_amdgcn_sched_barrier(0);
     // ---- compute phase --------------------------------------------------------------------------------------------
     __builtin_amdgcn_s_setprio(1);
@@ -191,7 +195,9 @@ __device__ __forceinline__ void gemm_tile_pingpong_mixed(const bf16_bits* __rest
     }
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);
+    RD_MARK(2);
     __builtin_amdgcn_s_barrier();
+    RD_MARK(3);
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -200,8 +206,10 @@ __device__ __forceinline__ void gemm_tile_pingpong_mixed(const bf16_bits* __rest
     if (p + 1 < nk) phase(p + 1, pp_detail::Parity<1>{});
   }
   if (group == 0) __builtin_amdgcn_s_barrier();
+  RD_MARK(4);
 
   store_accumulators<C>(acc, wm, wn, wave, lane, a_lim, b_lim, Op, ldo, smem);
+  RD_MARK(5);
 }
 
 }  // namespace rd
