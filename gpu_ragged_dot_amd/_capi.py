@@ -50,16 +50,19 @@ class VariantInfo(ctypes.Structure):
     ]
 
 
+ABI_VERSION = 2  # RD_ABI_VERSION of include/ragged_dot_hip.h this file mirrors
+
+
 class Plan(ctypes.Structure):
     _fields_ = [("variant", ctypes.c_int), ("group_m", ctypes.c_int), ("group_n", ctypes.c_int),
-                ("decode_nb", ctypes.c_int)]
+                ("decode_nb", ctypes.c_int), ("split_k", ctypes.c_int)]
 
-    def __init__(self, variant=-1, group_m=0, decode_nb=0, group_n=0):
-        super().__init__(variant, group_m, group_n, decode_nb)
+    def __init__(self, variant=-1, group_m=0, decode_nb=0, group_n=0, split_k=0):
+        super().__init__(variant, group_m, group_n, decode_nb, split_k)
 
     def __repr__(self):
         return (f"Plan(variant={self.variant}, group_m={self.group_m}, group_n={self.group_n}, "
-                f"decode_nb={self.decode_nb})")
+                f"decode_nb={self.decode_nb}, split_k={self.split_k})")
 
 
 # every symbol the header declares; checked at load time
@@ -90,6 +93,8 @@ def _load() -> ctypes.CDLL:
             raise ImportError(f"{LIB_PATH} does not export {name}")
     vp, ip, i, sz = ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
     lib.rd_abi_version.restype = i
+    if lib.rd_abi_version() != ABI_VERSION:
+        raise ImportError(f"{LIB_PATH} has ABI version {lib.rd_abi_version()}, this binding is for {ABI_VERSION}: rebuild it")
     lib.rd_last_error.restype = ctypes.c_char_p
     lib.rd_num_variants.restype = i
     lib.rd_get_variant.argtypes = [i, ctypes.POINTER(VariantInfo)]

@@ -27,7 +27,8 @@ struct DldsCfg {
   typedef bf16_bits Elem;
   static constexpr bool F32 = false;
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
-  static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = true, DLDS = true, PINGPONG = PINGPONG_, MIXED = false;
+  static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = true, DLDS = true, PINGPONG = PINGPONG_, MIXED = false,
+                        SPLITK = true;
   static constexpr int NW = WAVES_M * WAVES_N;
   static constexpr int NT = 64 * NW;
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
@@ -169,6 +170,65 @@ struct DldsFragReader {
   }
 };
 
+// One tile's contraction range cut into `parts` pieces that different work-groups compute.  Every piece drops its fp32
+// accumulators into its slot of `partials` and bumps the tile's arrival counter; the piece that arrives last sums all
+// pieces and is the one that stores the tile.  No work-group ever waits for another.
+struct SplitK {
+  float* partials = nullptr;    // [parts][NT * accumulators per thread] of this tile
+  int32_t* counter = nullptr;   // arrivals so far; zero when the launch starts
+  int parts = 1, part = 0;
+};
+
+// Returns true when the caller holds the complete sums and must store them.  All threads of the work-group call it,
+// after the last barrier of the K loop (it uses the first bytes of LDS to broadcast the arrival index).
+template <class C>
+__device__ __forceinline__ bool splitk_combine(f32x16_t (&acc)[C::TM][C::TN], const SplitK& sk, int tid,
+                                               unsigned char* smem) {
+  if (sk.parts <= 1) return true;
+  constexpr int QUADS = C::TM * C::TN * 4;  // float4 per thread
+  f32x4_t* mine = reinterpret_cast<f32x4_t*>(sk.partials) + (size_t)sk.part * (QUADS * C::NT) + tid;
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4_t v;
+        v[0] = acc[i][j][4 * g + 0]; v[1] = acc[i][j][4 * g + 1]; v[2] = acc[i][j][4 * g + 2]; v[3] = acc[i][j][4 * g + 3];
+        mine[((i * C::TN + j) * 4 + g) * C::NT] = v;
+      }
+  __threadfence();  // the partial sums are visible device-wide before the arrival is
+  __syncthreads();
+  int32_t* slot = reinterpret_cast<int32_t*>(smem);
+  if (tid == 0) *slot = atomicAdd(sk.counter, 1);
+  __syncthreads();
+  const int arrived = *slot;
+  __syncthreads();  // everyone has read the slot before the epilogue reuses LDS
+  if (arrived != sk.parts - 1) return false;
+  __threadfence();  // see the other pieces' stores, not stale cache lines
+  // Sum the pieces in index order, this work-group's own included, so that the result does not depend on which piece
+  // happened to arrive last.
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  for (int s = 0; s < sk.parts; ++s) {
+    const f32x4_t* other = reinterpret_cast<const f32x4_t*>(sk.partials) + (size_t)s * (QUADS * C::NT) + tid;
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+      for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const f32x4_t v = other[((i * C::TN + j) * 4 + g) * C::NT];
+          acc[i][j][4 * g + 0] += v[0]; acc[i][j][4 * g + 1] += v[1]; acc[i][j][4 * g + 2] += v[2]; acc[i][j][4 * g + 3] += v[3];
+        }
+  }
+  return true;
+}
+
 // Epilogue shared by the direct-to-LDS cores.  The matrix-core calls pass the B fragment as first operand, so the
 // accumulators hold transposed 32x32 blocks: register v of lane l is C[l & 31][8*(v>>2) + 4*(l>>5) + (v&3)], i.e. four
 // consecutive columns of one row per register quad.  Each wave drops its [WM][WN] patch into its own LDS area as bf16
@@ -208,7 +268,8 @@ __device__ __forceinline__ void store_accumulators(const f32x16_t (&acc)[C::TM][
 template <class C>
 __device__ __forceinline__ void gemm_tile_dlds(const bf16_bits* __restrict__ Ap, int lda, int a_lim,
                                                const bf16_bits* __restrict__ Bp, int ldb, int b_lim, int klen,
-                                               bf16_bits* __restrict__ Op, int ldo, bf16_bits* smem_) {
+                                               bf16_bits* __restrict__ Op, int ldo, bf16_bits* smem_,
+                                               const SplitK& sk = SplitK()) {
   RD_MARK_DECL;
   unsigned char* smem = reinterpret_cast<unsigned char*>(smem_);
   const int tid = threadIdx.x, lane = tid & 63;
@@ -313,6 +374,7 @@ __device__ __forceinline__ void gemm_tile_dlds(const bf16_bits* __restrict__ Ap,
   }
 
   __builtin_amdgcn_s_barrier();  // the ring is no longer read by any wave
+  if (!splitk_combine<C>(acc, sk, tid, smem)) return;
   store_accumulators<C>(acc, wm, wn, wave, lane, a_lim, b_lim, Op, ldo, smem);
 }
 
@@ -324,7 +386,8 @@ __device__ __forceinline__ void gemm_tile_dlds(const bf16_bits* __restrict__ Ap,
 template <class C>
 __device__ __forceinline__ void gemm_tile_pingpong(const bf16_bits* __restrict__ Ap, int lda, int a_lim,
                                                    const bf16_bits* __restrict__ Bp, int ldb, int b_lim, int klen,
-                                                   bf16_bits* __restrict__ Op, int ldo, bf16_bits* smem_) {
+                                                   bf16_bits* __restrict__ Op, int ldo, bf16_bits* smem_,
+                                               const SplitK& sk = SplitK()) {
   unsigned char* smem = reinterpret_cast<unsigned char*>(smem_);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -421,6 +484,7 @@ __device__ __forceinline__ void gemm_tile_pingpong(const bf16_bits* __restrict__
   }
   if (group == 0) __builtin_amdgcn_s_barrier();
 
+  if (!splitk_combine<C>(acc, sk, tid, smem)) return;
   store_accumulators<C>(acc, wm, wn, wave, lane, a_lim, b_lim, Op, ldo, smem);
 }
 

@@ -10,7 +10,8 @@ template <bool A_KMAJOR_, bool B_KMAJOR_>
 struct F32Cfg {
   typedef float Elem;
   static constexpr int BM = 64, BN = 64, BK = 16, WAVES_M = 2, WAVES_N = 2;
-  static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = false, DLDS = false, PINGPONG = false, MIXED = false;
+  static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = false, DLDS = false, PINGPONG = false, MIXED = false,
+                        SPLITK = false;
   static constexpr bool F32 = true;
   static constexpr int STAGES = 1;
   static constexpr int NT = 256, WAVES_PER_EU = 1;

@@ -14,7 +14,8 @@ struct PpCfg {
   typedef bf16_bits Elem;
   static constexpr bool F32 = false;
   static constexpr int BM = BM_, BN = BN_, BK = 32, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
-  static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = true, DLDS = true, PINGPONG = true, MIXED = true;
+  static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = true, DLDS = true, PINGPONG = true, MIXED = true,
+                        SPLITK = true;
   static constexpr int A_W = A_W_, A_S = A_S_, B_W = B_W_, B_S = B_S_;  // slab width (contraction), ring slots
   static constexpr int STAGES = A_S < B_S ? A_S : B_S;
   static constexpr int NW = WAVES_M * WAVES_N, NT = 64 * NW;
@@ -77,7 +78,7 @@ template <class C>
 __device__ __forceinline__ void gemm_tile_pingpong_mixed(const bf16_bits* __restrict__ Ap, int lda, int a_lim,
                                                          const bf16_bits* __restrict__ Bp, int ldb, int b_lim,
                                                          int klen, bf16_bits* __restrict__ Op, int ldo,
-                                                         bf16_bits* smem_) {
+                                                         bf16_bits* smem_, const SplitK& sk = SplitK()) {
   RD_MARK_DECL;
   unsigned char* smem = reinterpret_cast<unsigned char*>(smem_);
   const int tid = threadIdx.x, lane = tid & 63;
@@ -208,6 +209,7 @@ __device__ __forceinline__ void gemm_tile_pingpong_mixed(const bf16_bits* __rest
   if (group == 0) __builtin_amdgcn_s_barrier();
   RD_MARK(4);
 
+  if (!splitk_combine<C>(acc, sk, tid, smem)) return;
   store_accumulators<C>(acc, wm, wn, wave, lane, a_lim, b_lim, Op, ldo, smem);
   RD_MARK(5);
 }

@@ -22,7 +22,8 @@ struct TileCfg {
   typedef bf16_bits Elem;
   static constexpr bool F32 = false;
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
-  static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = VEC_, DLDS = false, PINGPONG = false, MIXED = false;
+  static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = VEC_, DLDS = false, PINGPONG = false, MIXED = false,
+                        SPLITK = false;
   static constexpr int STAGES = 2;
   static constexpr int NT = 64 * WAVES_M * WAVES_N;      // threads per work-group
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // per-wave tile

@@ -22,6 +22,12 @@ struct GmmArgs {
   int U;        // static bound on row tiles: ceil(m / BM) + g
   int n_tiles;  // ceil(n / BN)
   int group_m, group_n;  // tiles per L2-sharing block of the tile walk (rows x columns)
+  // K-split of the last, partly filled round of tiles (kernels whose configuration has SPLITK; 0 slots = off)
+  float* partials;     // [split_slots][BM * BN] fp32
+  int32_t* counters;   // [split_slots], zero at launch
+  int split_slots;     // work-groups appended to the launch for the split pieces
+  int num_cus;         // tiles the device runs at a time (one work-group per compute unit)
+  int main_grid;       // launch indices below this walk whole tiles (set by the launcher)
 };
 
 // dA[g, k, n] = x[rows of g, k]^T . dy[rows of g, n]
@@ -42,12 +48,36 @@ __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirs
 template <class C>
 __device__ __forceinline__ void run_tile(const typename C::Elem* Ap, int lda, int a_lim, const typename C::Elem* Bp,
                                          int ldb, int b_lim, int klen, typename C::Elem* Op, int ldo,
-                                         typename C::Elem* smem) {
+                                         typename C::Elem* smem, const SplitK& sk = SplitK()) {
   if constexpr (C::F32) gemm_tile_f32<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
-  else if constexpr (C::MIXED) gemm_tile_pingpong_mixed<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
-  else if constexpr (C::DLDS && C::PINGPONG) gemm_tile_pingpong<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
-  else if constexpr (C::DLDS) gemm_tile_dlds<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
+  else if constexpr (C::MIXED) gemm_tile_pingpong_mixed<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
+  else if constexpr (C::DLDS && C::PINGPONG) gemm_tile_pingpong<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
+  else if constexpr (C::DLDS) gemm_tile_dlds<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
   else gemm_tile<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
+}
+
+// How the last round of a gmm launch is cut along K.  The device runs num_cus tiles at a time; when the live tiles do
+// not fill the last round, the row tiles from `first_row` on (the ones that round would hold) are each computed by
+// `parts` work-groups over a `parts`-th of the contraction range instead, so the round takes about 1 / parts as long.
+struct SplitPlan {
+  int first_row;  // row tiles >= first_row are split; == total when nothing is
+  int parts;
+  int tiles;      // (total - first_row) * n_tiles
+};
+constexpr int kMaxSplitParts = 8;
+constexpr int kMinSplitK = 512;  // contraction elements a piece must keep
+
+__device__ __forceinline__ SplitPlan split_plan(int total, int n_tiles, int k, int slots, int num_cus) {
+  SplitPlan sp{total, 1, 0};
+  if (slots <= 0 || total <= 0) return sp;
+  const int live = total * n_tiles;
+  const int first = ((live / num_cus) * num_cus) / n_tiles;
+  const int tiles = (total - first) * n_tiles;
+  if (tiles <= 0) return sp;
+  int parts = imin(imin(slots / tiles, kMaxSplitParts), k / kMinSplitK);
+  if (parts < 2) return sp;
+  sp.first_row = first; sp.parts = parts; sp.tiles = tiles;
+  return sp;
 }
 
 // Walk tiles in bands of `group_m` rows: consecutive ids share B columns / A rows so that the ~32 tiles one XCD
@@ -73,17 +103,39 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
   // block's operand slabs are fetched into that XCD's L2 once), and blocks are dealt to the 8 XCDs (launch index mod 8)
   // round-robin.  Consecutive row tiles therefore spread over all XCDs, which keeps them evenly loaded when a few
   // groups are much longer than the rest and their tiles cost more than the mostly-empty ones.
-  const int per_block = p.group_m * p.group_n;
-  const int block_cols = (p.n_tiles + p.group_n - 1) / p.group_n;
-  const int pos = blockIdx.x >> 3;
-  const int block = (pos / per_block) * 8 + (blockIdx.x & 7);
-  const int q = pos % per_block;
-  const int mi = (block / block_cols) * p.group_m + q % p.group_m;
-  const int nj = (block % block_cols) * p.group_n + q / p.group_m;
-  if (mi >= p.U || nj >= p.n_tiles) return;
-
   // Everything read through the map is the same for the whole work-group: pin it to scalar registers.
   const int total = imin(uniform(*p.total_tiles), p.U);
+  SplitPlan sp{total, 1, 0};
+  if constexpr (C::SPLITK) sp = split_plan(total, p.n_tiles, p.k, p.split_slots, p.num_cus);
+
+  int mi, nj;
+  SplitK sk;
+  int k0 = 0, klen = p.k;
+  if ((int)blockIdx.x < p.main_grid) {
+    const int per_block = p.group_m * p.group_n;
+    const int block_cols = (p.n_tiles + p.group_n - 1) / p.group_n;
+    const int pos = blockIdx.x >> 3;
+    const int block = (pos / per_block) * 8 + (blockIdx.x & 7);
+    const int q = pos % per_block;
+    mi = (block / block_cols) * p.group_m + q % p.group_m;
+    nj = (block % block_cols) * p.group_n + q / p.group_m;
+    if (mi >= p.U || nj >= p.n_tiles) return;
+    if (mi >= sp.first_row && mi < total) return;  // computed in pieces by the appended work-groups
+  } else {
+    // piece `part` of split tile t; consecutive launch indices take consecutive tiles of one K range
+    const int r = blockIdx.x - p.main_grid;
+    if (r >= sp.tiles * sp.parts) return;
+    const int part = r / sp.tiles, t = r - part * sp.tiles;
+    mi = sp.first_row + t / p.n_tiles;
+    nj = t % p.n_tiles;
+    const int k64 = (p.k + 63) >> 6;
+    k0 = (int)((long long)k64 * part / sp.parts) << 6;
+    klen = imin(p.k, (int)((long long)k64 * (part + 1) / sp.parts) << 6) - k0;
+    sk.partials = p.partials + (size_t)t * sp.parts * (C::BM * C::BN);
+    sk.counter = p.counters + t;
+    sk.parts = sp.parts;
+    sk.part = part;
+  }
   const int col0 = nj * C::BN;
   const int cols = imin(C::BN, p.n - col0);
 
@@ -94,10 +146,11 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
     int rows = imin(C::BM, uniform(p.group_sizes[gi]) - it * C::BM);
     rows = imin(rows, p.m - row0);  // group_sizes summing past m: never touch rows >= m
     if (rows <= 0 || row0 < 0) return;
-    const E* Ap = px + (size_t)row0 * p.k;
-    const E* Bp = TRANS_RHS ? pA + (size_t)gi * p.n * p.k + (size_t)col0 * p.k : pA + (size_t)gi * p.k * p.n + col0;
+    const E* Ap = px + (size_t)row0 * p.k + k0;
+    const E* Bp = TRANS_RHS ? pA + (size_t)gi * p.n * p.k + (size_t)col0 * p.k + k0
+                            : pA + (size_t)gi * p.k * p.n + (size_t)k0 * p.n + col0;
     E* Op = py + (size_t)row0 * p.n + col0;
-    run_tile<C>(Ap, p.k, rows, Bp, TRANS_RHS ? p.k : p.n, cols, p.k, Op, p.n, smem);
+    run_tile<C>(Ap, p.k, rows, Bp, TRANS_RHS ? p.k : p.n, cols, klen, Op, p.n, smem, sk);
   } else {
     // Rows past sum(group_sizes) are defined to be zero.  The map never uses more than
     // U - ceil(tail / BM) entries, so the unused tile slots cover the tail.
@@ -156,6 +209,7 @@ struct TileVariant {
   int f32;     // 1: float32 operands and output; 0: bf16
   int dlds;    // 1: direct-to-LDS core (byte extents of one tile's operand window must stay below 2 GiB)
   int stages;  // LDS ring depth
+  int splitk;  // 1: the gmm kernels can cut the last round of tiles along K (needs partials in the workspace)
   gmm_launch_fn gmm_nn, gmm_nt;
   tgmm_launch_fn tgmm;
 };
@@ -172,9 +226,12 @@ int launch_gmm(hipStream_t s, const GmmArgs& a) {
   const int attr_rc = allow_big_lds(reinterpret_cast<const void*>(kern), C::LDS_BYTES);
   if (attr_rc != hipSuccess) return attr_rc;
   const int blocks = ((a.U + a.group_m - 1) / a.group_m) * ((a.n_tiles + a.group_n - 1) / a.group_n);
-  const int grid = 8 * ((blocks + 7) / 8) * a.group_m * a.group_n;
-  if (grid <= 0) return hipSuccess;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(C::NT), C::LDS_BYTES, s, a);
+  GmmArgs args = a;
+  args.main_grid = 8 * ((blocks + 7) / 8) * a.group_m * a.group_n;
+  if (!C::SPLITK) args.split_slots = 0;
+  const int grid = args.main_grid + args.split_slots;
+  if (args.main_grid <= 0) return hipSuccess;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(C::NT), C::LDS_BYTES, s, args);
   return (int)hipGetLastError();
 }
 

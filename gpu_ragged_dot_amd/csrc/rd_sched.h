@@ -7,9 +7,10 @@
 namespace rd {
 
 // Arrays as in the reference's GMMGroupLookupMetadata (gpu_ragged_dot.py:60-90); tile2group / tile2it hold
-// ceil(m / chunk) + g entries.
+// ceil(m / chunk) + g entries.  `counters` (may be null) are n_counters int32 cleared by the same launch.
 int launch_sched_map(hipStream_t s, const int32_t* group_sizes, int g, int m, int chunk, int32_t* group_offsets,
-                     int32_t* tile2group, int32_t* tile2it, int32_t* total_tiles);
+                     int32_t* tile2group, int32_t* tile2it, int32_t* total_tiles, int32_t* counters = nullptr,
+                     int n_counters = 0);
 
 // Stream-ordered clear that is safe to record into a HIP graph.
 int launch_zero_bytes(hipStream_t s, void* p, size_t bytes);

@@ -45,7 +45,10 @@ __global__ __launch_bounds__(kSchedThreads) void sched_map_kernel(const int32_t*
                                                                   int chunk, int32_t* __restrict__ group_offsets,
                                                                   int32_t* __restrict__ tile2group,
                                                                   int32_t* __restrict__ tile2it,
-                                                                  int32_t* __restrict__ total_tiles) {
+                                                                  int32_t* __restrict__ total_tiles,
+                                                                  int32_t* __restrict__ counters, int n_counters) {
+  // arrival counters of the K-split tiles of the launch that follows start at zero
+  for (int i = threadIdx.x; i < n_counters; i += kSchedThreads) counters[i] = 0;
   __shared__ uint32_t wave_a[kSchedWaves], wave_b[kSchedWaves];
   __shared__ int32_t incl[kSchedThreads];  // inclusive tile-count scan of the current slab of groups
   const int tid = threadIdx.x;
@@ -94,10 +97,10 @@ __global__ void fill_kernel(T* p, size_t n, T v) {
 }  // namespace
 
 int launch_sched_map(hipStream_t s, const int32_t* gs, int g, int m, int chunk, int32_t* group_offsets,
-                     int32_t* tile2group, int32_t* tile2it, int32_t* total_tiles) {
+                     int32_t* tile2group, int32_t* tile2it, int32_t* total_tiles, int32_t* counters, int n_counters) {
   const int U = (m + chunk - 1) / chunk + g;  // gpu_ragged_dot.py:77
   hipLaunchKernelGGL(sched_map_kernel, dim3(1), dim3(kSchedThreads), 0, s, gs, g, U, chunk, group_offsets,
-                     tile2group, tile2it, total_tiles);
+                     tile2group, tile2it, total_tiles, counters, counters ? n_counters : 0);
   return (int)hipGetLastError();
 }
 

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define RD_ABI_VERSION 1
+#define RD_ABI_VERSION 2
 
 enum rd_dtype { RD_DTYPE_BF16 = 0, RD_DTYPE_F32 = 1 };
 
@@ -55,6 +55,8 @@ typedef struct rd_plan {
   int group_m; /* tile walk: row tiles per L2-sharing block (tgmm: per band); 0 = default */
   int group_n; /* tile walk: column tiles per block (rd_gmm only); 0 = default */
   int decode_nb; /* rd_gmm only: > 0 selects the skinny-m streaming kernel with this many columns per work-group */
+  int split_k; /* rd_gmm only: 0 = when the tiles do not fill the device's last round, cut those tiles' contraction
+                  range over several work-groups (fp32 partial sums in the workspace); -1 = never */
 } rd_plan;
 
 int rd_abi_version(void);
@@ -83,7 +85,9 @@ int rd_sched_map_len(int m, int g, int chunk_m);
  *   A is [g, k, n] (trans_rhs = 0) or [g, n, k] (trans_rhs = 1, gpu_ragged_dot.py:139-144, :190).
  *   Rows of group i are [offset_i, offset_i + group_sizes[i]); rows >= sum(group_sizes) of y are set to zero
  *   (:155-165) -- also when every group is empty.  Groups that would run past m are clipped to m.
- * Workspace: rd_gmm_workspace_bytes() bytes, 256-byte aligned; holds the scheduling map. */
+ * Workspace: rd_gmm_workspace_bytes() bytes, 256-byte aligned; holds the scheduling map and, unless the plan says
+ * split_k = -1, fp32 partial sums (64 MiB for the 256 x 256 tiles).  A workspace that only has room for the map
+ * (the size returned for a plan with split_k = -1) is accepted: the call then runs without the K-split. */
 size_t rd_gmm_workspace_bytes(int m, int g, const rd_plan* plan /* host, may be NULL */);
 int rd_gmm(void* stream, const void* x, const void* A, const int32_t* group_sizes, void* y, int m, int k, int n,
            int g, int trans_rhs, int dtype, const rd_plan* plan /* host, may be NULL */, void* workspace,

@@ -146,6 +146,49 @@ def test_every_variant(vid, vname, vec, shape):
     assert not np.any(util.to_np(dA)[gs == 0])
 
 
+def _split_variants():
+    return [(v.id, v.name.decode()) for v in _capi.variants() if v.dtype == _capi.RD_DTYPE_BF16 and v.direct_to_lds]
+
+
+@pytest.mark.parametrize("trans_rhs", [False, True], ids=["A", "At"])
+@pytest.mark.parametrize("vid,vname", _split_variants(), ids=[v[1] for v in _split_variants()])
+@pytest.mark.parametrize("shape", [(900, 1096, 520, 5), (2100, 4104, 256, 3)], ids=["m900k1096n520g5", "m2100k4104n256g3"])
+def test_k_split_of_last_round(vid, vname, shape, trans_rhs):
+    """Few tiles and a long contraction: the tiles are cut along K over several work-groups.  The result must match
+    the oracle, agree with the unsplit run to fp32 summation order, overwrite every output element, and be the same on
+    a second call that reuses the workspace (the arrival counters are cleared by every call)."""
+    m, k, n, g = shape
+    print(f"k-split variant {vname} shape {shape} trans_rhs {trans_rhs}", flush=True)
+    lhs, rhs, _, gs, target_m = util.make_case(5, m, k, n, g, 0.9, True, scale_rhs=True)
+    gs[1] = 0
+    target_m = int(gs.sum())
+    x = util.bf16_dev(lhs)
+    A = util.bf16_dev(np.ascontiguousarray(np.swapaxes(rhs, 1, 2)) if trans_rhs else rhs)
+    gs_d = torch.from_numpy(gs).cuda()
+    split, whole = _capi.Plan(vid, 2, 0, 2, split_k=0), _capi.Plan(vid, 2, 0, 2, split_k=-1)
+    need = _capi.lib.rd_gmm_workspace_bytes(m, g, ctypes.byref(split))
+    assert need > _capi.lib.rd_gmm_workspace_bytes(m, g, ctypes.byref(whole))
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    ws.fill_(0xA5)  # stale counters and partial sums
+    outs = []
+    for plan in (split, split, whole):
+        y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        rc = _capi.lib.rd_gmm(torch.cuda.current_stream().cuda_stream, x.data_ptr(), A.data_ptr(), gs_d.data_ptr(),
+                              y.data_ptr(), m, k, n, g, int(trans_rhs), _capi.RD_DTYPE_BF16, ctypes.byref(plan),
+                              ws.data_ptr(), ws.numel())
+        torch.cuda.synchronize()
+        assert rc == 0, _capi.lib.rd_last_error()
+        outs.append(util.to_np(y))
+    y_ref = oracle.gmm(lhs, rhs, gs)
+    for y in outs:
+        assert not np.isnan(y).any()
+        util.assert_close_rows(y, y_ref, target_m, util.BF16_EPS, "y")
+        assert not np.any(y[target_m:])
+    assert np.array_equal(outs[0], outs[1])
+    scale = np.abs(y_ref).max()
+    assert np.abs(outs[0].astype(np.float32) - outs[2].astype(np.float32)).max() <= 2 ** -7 * scale
+
+
 # ---------------------------------------------------------------------------------------------------------------------
 # configuration C1 (tiny) with its exact recipe, and the other configurations' shapes
 # ---------------------------------------------------------------------------------------------------------------------
