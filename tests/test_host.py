@@ -90,6 +90,17 @@ def test_workspace_and_map_sizes():
             U = -(-m // v.tile_m) + g
             assert need >= (g + 2 * U + 1) * 4
         assert lib.rd_tgmm_workspace_bytes(m, g, None) >= (g + 2 * (g + 1) + 1) * 4
+        # the K-split of the last round needs 256 slots of tile_m x tile_n fp32 on top of the map; split_k = -1 and
+        # variants without it only need the map
+        import ctypes
+        whole = lib.rd_gmm_workspace_bytes(m, g, ctypes.byref(_capi.Plan(-1, split_k=-1)))
+        assert whole < (1 << 20) and need >= whole
+        for v in _capi.variants():
+            split = lib.rd_gmm_workspace_bytes(m, g, ctypes.byref(_capi.Plan(v.id)))
+            extra = 256 * 4 + 256 * v.tile_m * v.tile_n * 4
+            assert split in (whole, whole + extra), (v.name, split, whole)
+            if v.direct_to_lds:
+                assert split == whole + extra and need >= split
 
 
 def test_planner_block_rules_match_the_oracle():
