@@ -266,6 +266,36 @@ def test_every_output_element_is_written(fill_in):
         assert not np.any(y[target_m:])
 
 
+def test_degenerate_shapes():
+    """Empty contraction, no rows, a single narrow column block, more groups than the map kernel has threads, one
+    group, every group empty: the op is defined for all of them (zeros where nothing contributes)."""
+    rng = np.random.default_rng(0)
+    cases = [(64, 0, 64, 4, np.array([10, 20, 4, 30], np.int32)),
+             (0, 64, 64, 4, np.zeros(4, np.int32)),
+             (300, 64, 8, 3, np.array([100, 50, 150], np.int32)),
+             (5000, 128, 256, 3000, np.random.default_rng(1).multinomial(5000, [1 / 3000] * 3000).astype(np.int32)),
+             (2048, 256, 256, 1, np.array([2048], np.int32)),
+             (1024, 64, 128, 8, np.zeros(8, np.int32))]
+    for m, k, n, g, gs in cases:
+        print(f"degenerate m={m} k={k} n={n} g={g}", flush=True)
+        x = oracle.round_to(rng.standard_normal((m, k)).astype(np.float32), "bfloat16")
+        A = oracle.round_to((rng.standard_normal((g, k, n)) / max(k, 1) ** 0.5).astype(np.float32), "bfloat16")
+        dout = oracle.round_to(rng.standard_normal((m, n)).astype(np.float32), "bfloat16")
+        gs_t = torch.from_numpy(gs)
+        y = util.to_np(rd.ragged_dot(util.bf16_dev(x), util.bf16_dev(A), gs_t))
+        total = min(int(gs.sum()), m)
+        assert y.shape == (m, n) and not np.any(y[total:])
+        if y.size:
+            ref = oracle.gmm(x, A, gs)
+            assert np.abs(y - ref).max() <= 1e-2 * max(np.abs(ref).max(), 1e-30) + 0.0
+        dA = util.to_np(rd.trans_ragged_dot(util.bf16_dev(x), util.bf16_dev(dout), gs_t))
+        assert dA.shape == (g, k, n)
+        if dA.size:
+            ref = oracle.tgmm(x, dout, gs)
+            assert np.abs(dA - ref).max() <= 1e-2 * max(np.abs(ref).max(), 1e-30)
+            assert not np.any(dA[gs == 0])
+
+
 def test_group_sizes_past_m_are_clipped():
     """sum(group_sizes) > m is out-of-bounds in the reference; here rows >= m are never touched."""
     print("clip", flush=True)
