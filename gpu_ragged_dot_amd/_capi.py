@@ -78,6 +78,11 @@ EXPORTS = (
     "rd_gmm",
     "rd_tgmm_workspace_bytes",
     "rd_tgmm",
+    "rd_moe_route_workspace_bytes",
+    "rd_moe_route",
+    "rd_moe_dispatch",
+    "rd_moe_combine",
+    "rd_moe_combine_wgrad",
 )
 
 
@@ -113,6 +118,16 @@ def _load() -> ctypes.CDLL:
     lib.rd_tgmm_workspace_bytes.restype = sz
     lib.rd_tgmm.argtypes = [vp, vp, vp, ip, vp, i, i, i, i, i, ctypes.POINTER(Plan), vp, sz]
     lib.rd_tgmm.restype = i
+    lib.rd_moe_route_workspace_bytes.argtypes = [i, i, i]
+    lib.rd_moe_route_workspace_bytes.restype = sz
+    lib.rd_moe_route.argtypes = [vp, ip, i, i, i, ip, ip, ip, vp, sz]
+    lib.rd_moe_route.restype = i
+    lib.rd_moe_dispatch.argtypes = [vp, vp, ip, vp, vp, i, i, i, i]
+    lib.rd_moe_dispatch.restype = i
+    lib.rd_moe_combine.argtypes = [vp, vp, ip, vp, vp, i, i, i, i]
+    lib.rd_moe_combine.restype = i
+    lib.rd_moe_combine_wgrad.argtypes = [vp, vp, vp, ip, vp, i, i, i, i]
+    lib.rd_moe_combine_wgrad.restype = i
     return lib
 
 

@@ -101,6 +101,33 @@ int rd_tgmm(void* stream, const void* x, const void* dy, const int32_t* group_si
             int n, int g, int dtype, const rd_plan* plan /* host, may be NULL */, void* workspace,
             size_t workspace_bytes);
 
+/* ---- token routing around ragged_dot --------------------------------------------------------------------------
+ * The reference takes rows that are already sorted by group and leaves the sorting to its caller (its tests and
+ * tuner build sorted rows directly: tests.py:51-71, tuning.py:41-47).  These entry points are that caller's side for a
+ * mixture of experts, on the device, so that group_sizes is produced where rd_gmm consumes it.
+ *   A "slot" is one (token, choice) pair, numbered token * top_k + choice; a "row" is a row of the sorted matrix.
+ *   expert_ids[tokens * top_k]: expert of every slot; ids outside [0, g) mark dropped slots.
+ *   rd_moe_route: stable counting sort of the kept slots by expert id (ties keep slot order):
+ *     group_sizes[g]; row_of_slot[slots] (-1 for dropped slots); slot_of_row[slots] (-1 for rows past
+ *     sum(group_sizes)).  Bit-exact integer outputs.  1 <= g <= 12288, 1 <= top_k <= 64.
+ *   rd_moe_dispatch: x[row, :] = h[slot_of_row[row] / top_k, :] (times row_scale[slot] when row_scale is not NULL,
+ *     product rounded once to the element type); rows with slot -1 are zero.  h is [tokens, d], x is [slots, d].
+ *     With row_scale it is also the adjoint of rd_moe_combine with respect to y.
+ *   rd_moe_combine: out[token, :] = sum over its kept slots, in slot order, of weights[slot] * y[row_of_slot[slot], :]
+ *     (weights NULL = 1), fp32 accumulation, rounded once.  y is [slots, d], out is [tokens, d].  With weights NULL it
+ *     is the adjoint of rd_moe_dispatch.
+ *   rd_moe_combine_wgrad: dw[slot] = <y[row_of_slot[slot], :], dout[token, :]> in fp32 (0 for dropped slots).
+ * weights, row_scale and dw are float32 [tokens * top_k]. */
+size_t rd_moe_route_workspace_bytes(int tokens, int top_k, int g);
+int rd_moe_route(void* stream, const int32_t* expert_ids, int tokens, int top_k, int g, int32_t* group_sizes,
+                 int32_t* row_of_slot, int32_t* slot_of_row, void* workspace, size_t workspace_bytes);
+int rd_moe_dispatch(void* stream, const void* h, const int32_t* slot_of_row, const float* row_scale, void* x,
+                    int tokens, int top_k, int d, int dtype);
+int rd_moe_combine(void* stream, const void* y, const int32_t* row_of_slot, const float* weights, void* out,
+                   int tokens, int top_k, int d, int dtype);
+int rd_moe_combine_wgrad(void* stream, const void* y, const void* dout, const int32_t* row_of_slot, float* dw,
+                         int tokens, int top_k, int d, int dtype);
+
 #ifdef __cplusplus
 }
 #endif
