@@ -122,7 +122,7 @@ def _load() -> ctypes.CDLL:
     lib.rd_moe_route_workspace_bytes.restype = sz
     lib.rd_moe_route.argtypes = [vp, ip, i, i, i, ip, ip, ip, vp, sz]
     lib.rd_moe_route.restype = i
-    lib.rd_moe_dispatch.argtypes = [vp, vp, ip, vp, vp, i, i, i, i]
+    lib.rd_moe_dispatch.argtypes = [vp, vp, ip, ip, vp, vp, i, i, i, i]
     lib.rd_moe_dispatch.restype = i
     lib.rd_moe_combine.argtypes = [vp, vp, ip, vp, vp, i, i, i, i]
     lib.rd_moe_combine.restype = i

@@ -15,20 +15,19 @@ namespace rd {
 
 namespace {
 
-constexpr int kChunk = 2048;       // slots per single-wave work-group of the histogram and ranking kernels
 constexpr int kScanThreads = 1024;
 
 // ---- route -----------------------------------------------------------------------------------------------------------
 
 // hist[b][e] = number of kept slots of chunk b that go to expert e.
-__global__ __launch_bounds__(64) void moe_hist_kernel(const int32_t* __restrict__ ids, int S, int g,
+__global__ __launch_bounds__(64) void moe_hist_kernel(const int32_t* __restrict__ ids, int S, int g, int chunk,
                                                       int32_t* __restrict__ hist) {
   extern __shared__ int32_t cnt[];
   const int lane = threadIdx.x, b = blockIdx.x;
   for (int e = lane; e < g; e += 64) cnt[e] = 0;
   __syncthreads();
-  const int end = imin(S, (b + 1) * kChunk);
-  for (int s = b * kChunk + lane; s < end; s += 64) {
+  const int end = (int)(((long long)(b + 1) * chunk < S) ? (long long)(b + 1) * chunk : S);
+  for (int s = b * chunk + lane; s < end; s += 64) {
     const int e = ids[s];
     if (e >= 0 && e < g) atomicAdd(&cnt[e], 1);
   }
@@ -51,10 +50,15 @@ __global__ __launch_bounds__(kScanThreads) void moe_scan_kernel(int32_t* __restr
     const int e = base + tid;
     int total = 0;
     if (e < g) {
-      for (int b = 0; b < nb; ++b) {
-        const int32_t c = hist[(size_t)b * g + e];
-        hist[(size_t)b * g + e] = total;
-        total += c;
+      for (int b0 = 0; b0 < nb; b0 += 8) {  // eight independent loads at a time, then their running sums
+        int32_t c[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) c[u] = b0 + u < nb ? hist[(size_t)(b0 + u) * g + e] : 0;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (b0 + u < nb) hist[(size_t)(b0 + u) * g + e] = total;
+          total += c[u];
+        }
       }
       group_sizes[e] = total;
     }
@@ -80,7 +84,7 @@ __global__ __launch_bounds__(kScanThreads) void moe_scan_kernel(int32_t* __restr
 
 // Stable rank of every slot inside its chunk, chunk by 64 slots at a time: lanes of one expert find each other with
 // one ballot per id bit; the expert's running position lives in LDS.
-__global__ __launch_bounds__(64) void moe_rank_kernel(const int32_t* __restrict__ ids, int S, int g, int id_bits,
+__global__ __launch_bounds__(64) void moe_rank_kernel(const int32_t* __restrict__ ids, int S, int g, int chunk, int id_bits,
                                                       const int32_t* __restrict__ hist,
                                                       const int32_t* __restrict__ group_first,
                                                       int32_t* __restrict__ row_of_slot,
@@ -89,9 +93,9 @@ __global__ __launch_bounds__(64) void moe_rank_kernel(const int32_t* __restrict_
   const int lane = threadIdx.x, b = blockIdx.x;
   for (int e = lane; e < g; e += 64) pos[e] = group_first[e] + hist[(size_t)b * g + e];
   __syncthreads();
-  const int end = imin(S, (b + 1) * kChunk);
+  const int end = (int)(((long long)(b + 1) * chunk < S) ? (long long)(b + 1) * chunk : S);
   const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-  for (int s0 = b * kChunk; s0 < end; s0 += 64) {
+  for (int s0 = b * chunk; s0 < end; s0 += 64) {
     const int s = s0 + lane;
     const int e = s < end ? ids[s] : -1;
     const bool keep = e >= 0 && e < g;
@@ -122,39 +126,67 @@ template <> __device__ __forceinline__ float from_f32<float>(float v) { return v
 
 constexpr int kRowThreads = 256;
 
-// x[row] = h[slot / top_k] * scale[slot]; VEC: rows are whole 16-byte pieces at 16-byte aligned addresses.
+// x[row_of_slot[t, s]] = h[t] * scale[t, s] for every kept slot of token t: the token's row is read once and written
+// top_k times.  The rows past sum(group_sizes) (slot_of_row = -1) are zeroed by the work-group that owns their index
+// (row r belongs to work-group r / top_k for this purpose only).  VEC: rows are whole 16-byte pieces at 16-byte
+// aligned addresses.
 template <class T, bool VEC>
 __global__ __launch_bounds__(kRowThreads) void moe_dispatch_kernel(const T* __restrict__ h,
+                                                                   const int32_t* __restrict__ row_of_slot,
                                                                    const int32_t* __restrict__ slot_of_row,
                                                                    const float* __restrict__ row_scale, T* __restrict__ x,
                                                                    int top_k, int d) {
-  const int row = blockIdx.x, tid = threadIdx.x;
-  const int slot = __builtin_amdgcn_readfirstlane(slot_of_row[row]);
-  T* dst = x + (size_t)row * d;
+  __shared__ int32_t rows[kMoeMaxTopK];
+  __shared__ int32_t zero_row[kMoeMaxTopK];
+  __shared__ float sc[kMoeMaxTopK];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  if (tid < top_k) {
+    const size_t slot = (size_t)t * top_k + tid;
+    rows[tid] = row_of_slot[slot];
+    sc[tid] = row_scale ? row_scale[slot] : 1.f;
+    zero_row[tid] = slot_of_row[slot] < 0 ? (int32_t)slot : -1;
+  }
+  __syncthreads();
   constexpr int PER = 16 / sizeof(T);
-  if (slot < 0) {  // a row past sum(group_sizes): defined as zero
-    if (VEC) for (int c = tid; c < d / PER; c += kRowThreads) reinterpret_cast<u32x4_t*>(dst)[c] = u32x4_t{0, 0, 0, 0};
-    else for (int c = tid; c < d; c += kRowThreads) dst[c] = from_f32<T>(0.f);
-    return;
-  }
-  const T* src = h + (size_t)(slot / top_k) * d;
-  if (row_scale == nullptr) {
-    if (VEC) for (int c = tid; c < d / PER; c += kRowThreads)
-      reinterpret_cast<u32x4_t*>(dst)[c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(src) + c);
-    else for (int c = tid; c < d; c += kRowThreads) dst[c] = src[c];
-    return;
-  }
-  const float sc = row_scale[slot];
+  const T* src = h + (size_t)t * d;
   if (VEC) {
-    for (int c = tid; c < d / PER; c += kRowThreads) {
-      alignas(16) T v[PER];
-      *reinterpret_cast<u32x4_t*>(v) = reinterpret_cast<const u32x4_t*>(src)[c];
+    const int pieces = d / PER;
+    for (int c0 = tid; c0 < pieces; c0 += 4 * kRowThreads) {
+      u32x4_t v[4];
 #pragma unroll
-      for (int e = 0; e < PER; ++e) v[e] = from_f32<T>(to_f32<T>(v[e]) * sc);
-      reinterpret_cast<u32x4_t*>(dst)[c] = *reinterpret_cast<u32x4_t*>(v);
+      for (int u = 0; u < 4; ++u)  // clamped: always a valid piece, stored only if in range
+        v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(src) + imin(c0 + u * kRowThreads, pieces - 1));
+      for (int s = 0; s < top_k; ++s) {
+        if (rows[s] < 0) continue;
+        u32x4_t* dst = reinterpret_cast<u32x4_t*>(x + (size_t)rows[s] * d);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          if (c0 + u * kRowThreads >= pieces) continue;
+          u32x4_t o = v[u];
+          if (row_scale) {
+            alignas(16) T e[PER];
+            *reinterpret_cast<u32x4_t*>(e) = o;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) e[i] = from_f32<T>(to_f32<T>(e[i]) * sc[s]);
+            o = *reinterpret_cast<u32x4_t*>(e);
+          }
+          dst[c0 + u * kRowThreads] = o;
+        }
+      }
     }
+    for (int s = 0; s < top_k; ++s)
+      if (zero_row[s] >= 0)
+        for (int c = tid; c < pieces; c += kRowThreads)
+          reinterpret_cast<u32x4_t*>(x + (size_t)zero_row[s] * d)[c] = u32x4_t{0, 0, 0, 0};
   } else {
-    for (int c = tid; c < d; c += kRowThreads) dst[c] = from_f32<T>(to_f32<T>(src[c]) * sc);
+    for (int c = tid; c < d; c += kRowThreads) {
+      const float v = to_f32<T>(src[c]);
+      for (int s = 0; s < top_k; ++s)
+        if (rows[s] >= 0) x[(size_t)rows[s] * d + c] = row_scale ? from_f32<T>(v * sc[s]) : src[c];
+    }
+    for (int s = 0; s < top_k; ++s)
+      if (zero_row[s] >= 0)
+        for (int c = tid; c < d; c += kRowThreads) x[(size_t)zero_row[s] * d + c] = from_f32<T>(0.f);
   }
 }
 
@@ -230,42 +262,52 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 
 }  // namespace
 
+// Slots per single-wave work-group of the histogram and ranking kernels: short chunks for parallelism, longer ones
+// when the per-chunk histograms ([chunks][g] int32 in the workspace) would get large.
+static int route_chunk(long long slots, int g) {
+  int chunk = 512;
+  while (((slots + chunk - 1) / chunk) * g > (4ll << 20) && chunk < (1 << 20)) chunk *= 2;
+  return chunk;
+}
+
 size_t moe_route_workspace_bytes(long long slots, int g) {
-  const long long nb = (slots + kChunk - 1) / kChunk;
+  const int chunk = route_chunk(slots, g);
+  const long long nb = (slots + chunk - 1) / chunk;
   return (size_t)(nb * g + g) * sizeof(int32_t);
 }
 
 int launch_moe_route(hipStream_t s, const int32_t* ids, int slots, int g, int32_t* group_sizes, int32_t* row_of_slot,
                      int32_t* slot_of_row, int32_t* workspace) {
-  const int nb = (slots + kChunk - 1) / kChunk;
+  const int chunk = route_chunk(slots, g);
+  const int nb = (slots + chunk - 1) / chunk;
   int32_t* hist = workspace;
   int32_t* group_first = workspace + (size_t)nb * g;
   int id_bits = 0;
   while ((1 << id_bits) < g) ++id_bits;
   const size_t lds = (size_t)g * sizeof(int32_t);
-  if (nb > 0) hipLaunchKernelGGL(moe_hist_kernel, dim3(nb), dim3(64), lds, s, ids, slots, g, hist);
+  if (nb > 0) hipLaunchKernelGGL(moe_hist_kernel, dim3(nb), dim3(64), lds, s, ids, slots, g, chunk, hist);
   hipLaunchKernelGGL(moe_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, hist, nb, g, slots, group_sizes, group_first,
                      slot_of_row);
   if (nb > 0)
-    hipLaunchKernelGGL(moe_rank_kernel, dim3(nb), dim3(64), lds, s, ids, slots, g, id_bits, hist, group_first,
+    hipLaunchKernelGGL(moe_rank_kernel, dim3(nb), dim3(64), lds, s, ids, slots, g, chunk, id_bits, hist, group_first,
                        row_of_slot, slot_of_row);
   return (int)hipGetLastError();
 }
 
 template <class T>
-static int dispatch_t(hipStream_t s, const void* h, const int32_t* slot_of_row, const float* row_scale, void* x,
-                      int slots, int top_k, int d) {
+static int dispatch_t(hipStream_t s, const void* h, const int32_t* row_of_slot, const int32_t* slot_of_row,
+                      const float* row_scale, void* x, int tokens, int top_k, int d) {
   const bool vec = (d * sizeof(T)) % 16 == 0 && aligned16(h) && aligned16(x);
-  if (vec) hipLaunchKernelGGL((moe_dispatch_kernel<T, true>), dim3(slots), dim3(kRowThreads), 0, s, (const T*)h, slot_of_row, row_scale, (T*)x, top_k, d);
-  else hipLaunchKernelGGL((moe_dispatch_kernel<T, false>), dim3(slots), dim3(kRowThreads), 0, s, (const T*)h, slot_of_row, row_scale, (T*)x, top_k, d);
+  if (vec) hipLaunchKernelGGL((moe_dispatch_kernel<T, true>), dim3(tokens), dim3(kRowThreads), 0, s, (const T*)h, row_of_slot, slot_of_row, row_scale, (T*)x, top_k, d);
+  else hipLaunchKernelGGL((moe_dispatch_kernel<T, false>), dim3(tokens), dim3(kRowThreads), 0, s, (const T*)h, row_of_slot, slot_of_row, row_scale, (T*)x, top_k, d);
   return (int)hipGetLastError();
 }
 
-int launch_moe_dispatch(hipStream_t s, const void* h, const int32_t* slot_of_row, const float* row_scale, void* x,
-                        int slots, int top_k, int d, bool f32) {
-  if (slots <= 0 || d <= 0) return hipSuccess;
-  return f32 ? dispatch_t<float>(s, h, slot_of_row, row_scale, x, slots, top_k, d)
-             : dispatch_t<bf16_bits>(s, h, slot_of_row, row_scale, x, slots, top_k, d);
+int launch_moe_dispatch(hipStream_t s, const void* h, const int32_t* row_of_slot, const int32_t* slot_of_row,
+                        const float* row_scale, void* x, int tokens, int top_k, int d, bool f32) {
+  if (tokens <= 0 || d <= 0) return hipSuccess;
+  return f32 ? dispatch_t<float>(s, h, row_of_slot, slot_of_row, row_scale, x, tokens, top_k, d)
+             : dispatch_t<bf16_bits>(s, h, row_of_slot, slot_of_row, row_scale, x, tokens, top_k, d);
 }
 
 template <class T>

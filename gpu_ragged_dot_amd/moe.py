@@ -68,7 +68,7 @@ def _dispatch(h, r: Routing, row_scale):
     d = h.shape[1]
     x = torch.empty((r.tokens * r.top_k, d), dtype=h.dtype, device=dev)
     with torch.cuda.device(dev):
-        _capi.check(_capi.lib.rd_moe_dispatch(_stream_ptr(dev), h.data_ptr(), r.slot_of_row.data_ptr(),
+        _capi.check(_capi.lib.rd_moe_dispatch(_stream_ptr(dev), h.data_ptr(), r.row_of_slot.data_ptr(), r.slot_of_row.data_ptr(),
                                               row_scale.data_ptr() if row_scale is not None else None, x.data_ptr(),
                                               r.tokens, r.top_k, d, _dtype(h)))
     return x

@@ -112,6 +112,7 @@ int rd_tgmm(void* stream, const void* x, const void* dy, const int32_t* group_si
  *     sum(group_sizes)).  Bit-exact integer outputs.  1 <= g <= 12288, 1 <= top_k <= 64.
  *   rd_moe_dispatch: x[row, :] = h[slot_of_row[row] / top_k, :] (times row_scale[slot] when row_scale is not NULL,
  *     product rounded once to the element type); rows with slot -1 are zero.  h is [tokens, d], x is [slots, d].
+ *     Takes both index arrays of rd_moe_route: each token's row is read once and written to its top_k rows.
  *     With row_scale it is also the adjoint of rd_moe_combine with respect to y.
  *   rd_moe_combine: out[token, :] = sum over its kept slots, in slot order, of weights[slot] * y[row_of_slot[slot], :]
  *     (weights NULL = 1), fp32 accumulation, rounded once.  y is [slots, d], out is [tokens, d].  With weights NULL it
@@ -121,8 +122,8 @@ int rd_tgmm(void* stream, const void* x, const void* dy, const int32_t* group_si
 size_t rd_moe_route_workspace_bytes(int tokens, int top_k, int g);
 int rd_moe_route(void* stream, const int32_t* expert_ids, int tokens, int top_k, int g, int32_t* group_sizes,
                  int32_t* row_of_slot, int32_t* slot_of_row, void* workspace, size_t workspace_bytes);
-int rd_moe_dispatch(void* stream, const void* h, const int32_t* slot_of_row, const float* row_scale, void* x,
-                    int tokens, int top_k, int d, int dtype);
+int rd_moe_dispatch(void* stream, const void* h, const int32_t* row_of_slot, const int32_t* slot_of_row,
+                    const float* row_scale, void* x, int tokens, int top_k, int d, int dtype);
 int rd_moe_combine(void* stream, const void* y, const int32_t* row_of_slot, const float* weights, void* out,
                    int tokens, int top_k, int d, int dtype);
 int rd_moe_combine_wgrad(void* stream, const void* y, const void* dout, const int32_t* row_of_slot, float* dw,
