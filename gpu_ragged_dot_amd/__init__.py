@@ -4,8 +4,9 @@
 (gpu_ragged_dot.py:30, 406, 454) computed by hand-written gfx950 kernels behind a C ABI.
 """
 
+from . import moe  # noqa: F401  (route / dispatch / combine around ragged_dot)
 from .ops import gmm, make_group_metadata, ragged_dot, ragged_dot_vjp, tgmm, trans_ragged_dot
 from .planner import CHUNK_M, DEFAULT_BLOCK_K, DEFAULT_BLOCK_M, DEFAULT_BLOCK_N
 
 __all__ = ["gmm", "tgmm", "ragged_dot", "trans_ragged_dot", "ragged_dot_vjp", "make_group_metadata",
-           "CHUNK_M", "DEFAULT_BLOCK_M", "DEFAULT_BLOCK_N", "DEFAULT_BLOCK_K"]
+           "moe", "CHUNK_M", "DEFAULT_BLOCK_M", "DEFAULT_BLOCK_N", "DEFAULT_BLOCK_K"]
