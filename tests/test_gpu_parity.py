@@ -382,3 +382,57 @@ def test_float32_trans_ragged_dot(c):
     ref = oracle.tgmm(lhs, dout, gs, out_dtype="float32", acc=np.float64)
     assert float(np.max(oracle.err_fn(util.to_np(out), ref, axis=(-1, -2), mask=gs != 0))) < F32_TGMM_EPS
     assert not np.any(util.to_np(out)[gs == 0])
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# HIP graph capture: no entry point reads device data on the host, so a captured step replays correctly
+# ---------------------------------------------------------------------------------------------------------------------
+
+def test_graph_capture_and_replay():
+    """Forward + both backward products (tile kernels with the K-split, the streaming kernel, the routing kernels)
+    captured once and replayed with new inputs in the same buffers: every replay must equal the eager result of the
+    same inputs, with eager work and synchronisation in between."""
+    from gpu_ragged_dot_amd import moe, ops
+    print("graph capture", flush=True)
+    hp = dict(block_m=64, block_k=64, block_n=64, interpret=False, compute_dtype=None, acc_dtype=torch.float32, chunk_m=512)
+    m, k, n, g = 1500, 1096, 520, 6           # few tiles, long contraction: the K-split engages on the big tiles
+    tokens, top_k = 750, 2
+    gen = torch.Generator(device="cuda").manual_seed(0)
+
+    def fresh():
+        h = torch.randn((tokens, k), generator=gen, device="cuda").to(torch.bfloat16)
+        A = (torch.randn((g, k, n), generator=gen, device="cuda") / k ** 0.5).to(torch.bfloat16)
+        dout = torch.randn((m, n), generator=gen, device="cuda").to(torch.bfloat16)
+        ids = torch.randint(0, g, (tokens, top_k), generator=gen, device="cuda", dtype=torch.int32)
+        return h, A, dout, ids
+
+    big = _capi.Plan([v.id for v in _capi.variants() if v.name.decode().startswith("q256")][0], 2, 0, 2)
+
+    def step(h, A, dout, ids):
+        r = moe.route(ids, g)
+        x = moe._dispatch(h, r, None)
+        y = ops._gmm_fwd(x, A, r.group_sizes, **hp, trans_rhs=False, plan=big)
+        dx = ops._gmm_fwd(dout, A, r.group_sizes, **hp, trans_rhs=True, plan=big)
+        dA = ops._tgmm_fwd(x, dout, r.group_sizes, **hp, plan=big)
+        y_small = ops._gmm_fwd(x[:64].contiguous(), A, torch.clamp(r.group_sizes, max=10), **hp, trans_rhs=False,
+                               plan=_capi.Plan(-1, 0, 64))
+        out = moe._combine(y, r, None)
+        return y, dx, dA, y_small, out
+
+    static = [t.clone() for t in fresh()]
+    step(*static)                              # warm-up: kernel attributes are set outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step(*static)
+    for _ in range(3):
+        new = fresh()
+        for dst, src in zip(static, new):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        want = step(*new)                      # eager, on the default stream
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
