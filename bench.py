@@ -215,6 +215,18 @@ def main():
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
 
+    # The decode step is one ~40 us launch: also time it replayed from a HIP graph (one graph = one call per weight
+    # copy), which takes the host's launch path out of the measurement.
+    graph_ms = None
+    if name == "decode":
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for a in copies:
+                ops._gmm_fwd(x, a, gs, **hp, trans_rhs=False)
+        for _ in range(3):
+            graph.replay()
+        graph_ms = _event_ms(graph.replay, max(args.steps // len(copies), 4), torch) / len(copies)
+
     # per-kernel launch durations, for the roofline of the dominant kernel
     per = {pname: _event_ms(fn, max(args.steps, 5), torch) for pname, fn in parts}
     dominant = max(per, key=per.get)
@@ -272,6 +284,7 @@ def main():
                    "description": w.description, "group_sizes": "seeded, see gpu_ragged_dot_amd/workloads.py"},
         "frac_of_bf16_mfma_peak": (value / PEAK_BF16_TFLOPS) if unit == "TFLOP/s" else None,
         "per_kernel_ms": per,
+        "graph_replay_ms_per_step": graph_ms,
         "tile_plans": plans,
         "wall_s_timed_region": wall,
         "roofline": roof,
