@@ -228,7 +228,10 @@ def main():
         graph_ms = _event_ms(graph.replay, max(args.steps // len(copies), 4), torch) / len(copies)
 
     # per-kernel launch durations, for the roofline of the dominant kernel
-    per = {pname: _event_ms(fn, max(args.steps, 5), torch) for pname, fn in parts}
+    if len(parts) == 1:  # the step is that one product: the timed region already is its launch duration
+        per = {parts[0][0]: ms_per_step}
+    else:
+        per = {pname: _event_ms(fn, max(args.steps, 5), torch) for pname, fn in parts}
     dominant = max(per, key=per.get)
     flops_step = workloads.flops(name)
     abytes = workloads.algorithmic_bytes(name)
@@ -257,7 +260,7 @@ def main():
             roof["traffic"] = json.load(f).get(name, {}).get(dominant)
     except (OSError, ValueError):
         pass
-    roof["kernel"] = {"fwd": "gmm_kernel<.., trans_rhs=false>" if name != "decode" else "gmm_decode_kernel",
+    roof["kernel"] = {"fwd": "gmm_kernel<.., trans_rhs=false>" if name != "decode" else "gmm_rows_kernel + gmm_rows_finish_kernel",
                       "dlhs": "gmm_kernel<.., trans_rhs=true>", "drhs": "tgmm_kernel"}[dominant]
     roof["launch_ms"] = per[dominant]
 
@@ -265,7 +268,7 @@ def main():
     for pname, op, (mm, kk, nn) in (("fwd", 0, (w.m, w.k, w.n)), ("dlhs", 1, (w.m, w.n, w.k)), ("drhs", 2, (w.m, w.k, w.n))):
         if pname in per:
             p = planner.select_plan(op, mm, kk, nn, w.g)
-            plans[pname] = ("decode_nb%d" % p.decode_nb) if p.decode_nb else planner.compiled_variants()[p.variant].name.decode()
+            plans[pname] = ("decode_rows" if p.decode_nb < 0 else "decode_nb%d" % p.decode_nb) if p.decode_nb else planner.compiled_variants()[p.variant].name.decode()
 
     out = {
         "metric": metric,

@@ -17,4 +17,11 @@ struct DecodeArgs {
 constexpr int kDecodeMaxK = 16384;
 int launch_gmm_decode(hipStream_t s, const DecodeArgs& a, int nb);
 
+// Whole-row slices: every non-empty expert's weights are cut into equally many contiguous pieces along k, one per
+// work-group; fp32 partial sums [m][pieces][n] in the workspace, a second kernel adds them.  Needs n % 8 == 0,
+// n <= 2048, k * n < 2^31 and a 16-byte aligned workspace of at least gmm_rows_workspace_bytes(m, n, 1) bytes (more
+// room = more pieces, up to what keeps ~3 work-groups per compute unit busy).
+size_t gmm_rows_workspace_bytes(int m, int n, int pieces);
+int launch_gmm_rows(hipStream_t s, const DecodeArgs& a, int num_cus, void* workspace, size_t workspace_bytes);
+
 }  // namespace rd

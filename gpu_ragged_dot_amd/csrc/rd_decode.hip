@@ -1,10 +1,14 @@
 // Forward ragged_dot for a handful of rows per group (token-by-token decoding through a mixture of experts).
 // The op is then a stream over the weights of the non-empty experts: each weight element is used by <= a few
-// rows, so the matrix cores are pointless and HBM bandwidth is everything.  One launch does the whole op: every
-// work-group finds its group's row range itself (a 128-entry sum), so no scheduling-map kernel runs first.
+// rows, so the matrix cores are pointless and HBM bandwidth is everything.  No scheduling-map kernel runs first:
+// every work-group finds its group's row range itself from the group sizes.
 //
-// Work-group (group gi, column block jb): streams A[gi][:, jb*NB .. +NB) once with 16-byte loads, ROWS rows of x at
-// a time held in LDS, fp32 accumulation on the vector ALU, one cross-lane + cross-wave reduction at the end.
+// Two ways of cutting the stream into work-groups:
+//  * gmm_decode_kernel<NB>: work-group (group gi, column block jb) streams A[gi][:, jb*NB .. +NB) over the whole
+//    contraction range and writes y itself - one launch, no workspace;
+//  * gmm_rows_kernel: work-group (non-empty group, slice of the contraction range) streams whole rows of A[gi] - equal
+//    contiguous blocks - and leaves fp32 partial sums for gmm_rows_finish_kernel (second half of this file).
+// Both hold ROWS rows of x at a time in LDS, accumulate in fp32 on the vector ALU and reduce across lanes at the end.
 #include "rd_common.h"
 #include "rd_decode.h"
 
@@ -208,6 +212,239 @@ int launch_nb(hipStream_t s, const DecodeArgs& a) {
   return (int)hipGetLastError();
 }
 
+
+// ---- whole-row slices ----------------------------------------------------------------------------------------------
+// The strip kernel above reads 64- to 256-byte pieces of every weight row and has as many work-groups as there are
+// (non-empty expert, column strip) pairs; on the decode shape that is 636 unequal-looking jobs for 256 compute units,
+// and bare load kernels show that this access pattern tops out ~25 % below what contiguous, evenly spread blocks
+// reach.  The kernel below cuts the stream the other way: every non-empty expert gets the same number C of
+// work-groups, each taking whole rows of the weight matrix for a C-th of the contraction range - one contiguous block
+// of memory, all blocks the same size.  A piece only yields partial sums: they go to the workspace as fp32
+// [row][C][n] and a second, tiny kernel adds the C pieces in order, rounds, and zeroes the rows past sum(group_sizes).
+// Which expert a work-group serves depends on which experts are non-empty, so every work-group first scans the group
+// sizes (from L2) - the one dependent step before its weight stream starts.
+
+constexpr int kRowsDepth = 6;  // 16-byte weight loads in flight per thread (measured: 3 -> 39 us, 4 -> 34.4, 6 -> 33.2, 8 -> 34.3, 16 -> 36.6)
+constexpr int kMaxSeg = 2048;  // contraction indices staged in LDS at a time
+
+struct RowsGeom {
+  int wgs;       // work-groups launched
+  int lpr;       // threads across one weight row = n / 8 (<= 256)
+  int rps;       // weight rows fetched per step = 256 / lpr
+  int max_c;     // most pieces per expert the workspace has room for
+  int min_rows;  // fewest contraction indices a piece may get
+};
+
+struct RowsHeader { int32_t pieces, total_rows; };  // written by work-group 0 for the finishing kernel
+
+__device__ __forceinline__ u32x4_t load_row_step(const bf16_bits* W, uint32_t coff, int step, int rps, int kr, int klen, int n) {
+  const int kk = imin(step * rps + kr, klen - 1);  // clamped, masked when consumed
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(W + (uint32_t)kk * (uint32_t)n + coff));
+}
+
+template <int R>
+__device__ __forceinline__ void fma_row_step(float (&acc)[kRows][8], const u32x4_t w, const u32x2_t* xs, int step, int rps,
+                                             int kr, int klen) {
+  const int kk_raw = step * rps + kr;
+  const uint32_t live = kk_raw < klen ? 0xffffffffu : 0u;
+  const u32x2_t xp = xs[imin(kk_raw, klen - 1)];
+  float xv[kRows];
+  xv[0] = __builtin_bit_cast(float, (xp[0] << 16) & live);
+  xv[1] = __builtin_bit_cast(float, xp[0] & 0xffff0000u & live);
+  xv[2] = __builtin_bit_cast(float, (xp[1] << 16) & live);
+  xv[3] = __builtin_bit_cast(float, xp[1] & 0xffff0000u & live);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float lo = __builtin_bit_cast(float, w[e] << 16);
+    const float hi = __builtin_bit_cast(float, w[e] & 0xffff0000u);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      acc[r][2 * e] = __builtin_fmaf(xv[r], lo, acc[r][2 * e]);
+      acc[r][2 * e + 1] = __builtin_fmaf(xv[r], hi, acc[r][2 * e + 1]);
+    }
+  }
+}
+
+template <int R>
+__device__ __forceinline__ void stream_rows(float (&acc)[kRows][8], u32x4_t (&w)[kRowsDepth], const bf16_bits* W, uint32_t coff,
+                                            const u32x2_t* xs, int rps, int kr, int klen, int n) {
+  const int nsteps = (klen + rps - 1) / rps;
+  for (int base = 0; base < nsteps; base += kRowsDepth) {
+#pragma unroll
+    for (int u = 0; u < kRowsDepth; ++u) {
+      fma_row_step<R>(acc, w[u], xs, base + u, rps, kr, klen);
+      w[u] = load_row_step(W, coff, base + kRowsDepth + u, rps, kr, klen, n);
+    }
+  }
+}
+
+__global__ __launch_bounds__(kThreads, 2) void gmm_rows_kernel(DecodeArgs p, RowsGeom q, RowsHeader* __restrict__ header,
+                                                               float* __restrict__ partials) {
+  __shared__ int32_t wave_cnt[2][kThreads / 64];
+  __shared__ int32_t job[3];                // expert, first row, rows of the expert this work-group serves
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  u32x2_t* xs = reinterpret_cast<u32x2_t*>(smem_raw);                   // [kMaxSeg] x {4 rows as bf16}
+  float* part = reinterpret_cast<float*>(smem_raw + kMaxSeg * 8);        // [rps][kRows][n]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+  // ---- which experts are non-empty, and where their rows start: a scan over the group sizes --------------------------
+  // One slab of kThreads experts at a time: every thread learns how many non-empty experts and rows precede its own.
+  // With g <= kThreads (the usual case) the group sizes are read once and the result stays in registers.
+  auto scan_slab = [&](int base, int seen, int rows_seen, int& sz, int& rank, int& first_row, int& slab_act, int& slab_rows) {
+    const int e = base + tid;
+    sz = e < p.g ? imax(p.group_sizes[e], 0) : 0;
+    const unsigned long long m_act = __ballot(sz > 0);
+    const int before_in_wave = __popcll(m_act & ((1ull << lane) - 1ull));
+    int incl = sz;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) { const int up = __shfl_up(incl, d, 64); if (lane >= d) incl += up; }
+    __syncthreads();  // wave_cnt free again
+    if (lane == 63) { wave_cnt[0][wave] = __popcll(m_act); wave_cnt[1][wave] = incl; }
+    __syncthreads();
+    rank = seen + before_in_wave;
+    first_row = rows_seen + incl - sz;
+    slab_act = 0; slab_rows = 0;
+    for (int w2 = 0; w2 < kThreads / 64; ++w2) {
+      if (w2 < wave) { rank += wave_cnt[0][w2]; first_row += wave_cnt[1][w2]; }
+      slab_act += wave_cnt[0][w2]; slab_rows += wave_cnt[1][w2];
+    }
+  };
+  const bool one_slab = p.g <= kThreads;
+  int sz0 = 0, rank0 = 0, first0 = 0;
+  int n_act = 0, total = 0;
+  for (int base = 0; base < p.g; base += kThreads) {
+    int sz, rank, first_row, sa, sr;
+    scan_slab(base, n_act, total, sz, rank, first_row, sa, sr);
+    if (base == 0) { sz0 = sz; rank0 = rank; first0 = first_row; }
+    n_act += sa; total += sr;
+  }
+  int C = n_act > 0 ? q.wgs / n_act : 1;
+  C = imax(1, imin(imin(C, q.max_c), p.k / q.min_rows));
+  if (blockIdx.x == 0 && tid == 0) { header->pieces = C; header->total_rows = imin(total, p.m); }
+  if (n_act == 0 || (int)blockIdx.x >= (q.wgs / C) * C) return;  // nothing to do / left-over work-groups
+
+  const int c = blockIdx.x % C;
+  for (int want = blockIdx.x / C; want < n_act; want += q.wgs / C) {
+    // the `want`-th non-empty expert and the rows before it
+    __syncthreads();  // job free again
+    if (one_slab) {
+      if (sz0 > 0 && rank0 == want) { job[0] = tid; job[1] = first0; job[2] = sz0; }
+    } else {
+      int seen = 0, rows_seen = 0;
+      for (int base = 0; base < p.g; base += kThreads) {
+        int sz, rank, first_row, sa, sr;
+        scan_slab(base, seen, rows_seen, sz, rank, first_row, sa, sr);
+        if (sz > 0 && rank == want) { job[0] = base + tid; job[1] = first_row; job[2] = sz; }
+        seen += sa; rows_seen += sr;
+      }
+    }
+    __syncthreads();
+    const int gi = job[0], row0 = job[1];
+    const int rows = imin(job[2], p.m - row0);
+    if (rows <= 0) continue;
+
+    // ---- this piece: contraction indices [k0, k0 + klen_all) of expert gi, whole rows ---------------------------------
+    const int unit = q.rps * 2;
+    const int per = ((p.k + C - 1) / C + unit - 1) / unit * unit;
+    const int k0 = c * per;
+    const int klen_all = imin(per, p.k - k0);
+    const int tc = tid % q.lpr, kr = tid / q.lpr;
+    const bool loader = kr < q.rps;
+    const uint32_t coff = (uint32_t)(tc * 8);
+    for (int rc = 0; rc < rows; rc += kRows) {
+      const int nr = imin(kRows, rows - rc);
+      float acc[kRows][8];
+#pragma unroll
+      for (int r = 0; r < kRows; ++r)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[r][e] = 0.f;
+      for (int s0 = 0; s0 < klen_all; s0 += kMaxSeg) {
+        const int klen = imin(kMaxSeg, klen_all - s0);
+        const bf16_bits* W = p.A + (size_t)gi * p.k * p.n + (size_t)(k0 + s0) * p.n;
+        u32x4_t w[kRowsDepth];
+        if (loader) {
+#pragma unroll
+          for (int u = 0; u < kRowsDepth; ++u) w[u] = load_row_step(W, coff, u, q.rps, kr, klen, p.n);
+        }
+        __syncthreads();  // previous segment / pass done with xs and part
+        for (int j = tid; j < klen; j += kThreads) {
+          uint32_t v[kRows];
+#pragma unroll
+          for (int r = 0; r < kRows; ++r) {
+            const uint32_t x = p.x[(size_t)(row0 + rc + imin(r, nr - 1)) * p.k + k0 + s0 + j];
+            v[r] = r < nr ? x : 0u;
+          }
+          xs[j] = u32x2_t{v[0] | (v[1] << 16), v[2] | (v[3] << 16)};
+        }
+        __syncthreads();
+        if (loader) {
+          switch (nr) {
+            case 1: stream_rows<1>(acc, w, W, coff, xs, q.rps, kr, klen, p.n); break;
+            case 2: stream_rows<2>(acc, w, W, coff, xs, q.rps, kr, klen, p.n); break;
+            case 3: stream_rows<3>(acc, w, W, coff, xs, q.rps, kr, klen, p.n); break;
+            default: stream_rows<4>(acc, w, W, coff, xs, q.rps, kr, klen, p.n); break;
+          }
+        }
+      }
+      // reduce over the rps row slots through LDS, then hand the piece's sums over
+      __syncthreads();
+      if (loader) {
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) {
+          float* dst = part + ((size_t)(kr * kRows + r) * p.n + tc * 8);
+          *reinterpret_cast<f32x4_t*>(dst) = f32x4_t{acc[r][0], acc[r][1], acc[r][2], acc[r][3]};
+          *reinterpret_cast<f32x4_t*>(dst + 4) = f32x4_t{acc[r][4], acc[r][5], acc[r][6], acc[r][7]};
+        }
+      }
+      __syncthreads();
+      for (int idx = tid; idx < nr * p.n; idx += kThreads) {
+        const int r = idx / p.n, col = idx - r * p.n;
+        float v = 0.f;
+        for (int s2 = 0; s2 < q.rps; ++s2) v += part[(size_t)(s2 * kRows + r) * p.n + col];
+        partials[((size_t)(row0 + rc + r) * C + c) * p.n + col] = v;
+      }
+    }
+  }
+}
+
+// y[row, :] = sum over the pieces of partials[row, piece, :] for rows below sum(group_sizes), zero above.
+// Work-group = (row, block of 256 columns); thread = (8 columns, one of 8 piece lanes).
+__global__ __launch_bounds__(kThreads) void gmm_rows_finish_kernel(DecodeArgs p, const RowsHeader* __restrict__ header,
+                                                                   const float* __restrict__ partials) {
+  __shared__ float sums[8][32][8];
+  const int tid = threadIdx.x;
+  const int col_blocks = (p.n + 255) / 256;
+  const int row = blockIdx.x / col_blocks, cb = blockIdx.x - row * col_blocks;
+  const int C = header->pieces, total = header->total_rows;
+  const int chunk = tid & 31, lane_s = tid >> 5;
+  const int col = cb * 256 + chunk * 8;
+  float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (row < total && col < p.n) {
+    for (int s = lane_s; s < C; s += 8) {
+      const f32x4_t* src = reinterpret_cast<const f32x4_t*>(partials + ((size_t)row * C + s) * p.n + col);
+      const f32x4_t a = src[0], b = src[1];
+      v[0] += a[0]; v[1] += a[1]; v[2] += a[2]; v[3] += a[3];
+      v[4] += b[0]; v[5] += b[1]; v[6] += b[2]; v[7] += b[3];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) sums[lane_s][chunk][e] = v[e];
+  __syncthreads();
+  if (lane_s == 0 && col < p.n) {
+    float t[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      t[e] = 0.f;
+#pragma unroll
+      for (int s = 0; s < 8; ++s) t[e] += sums[s][chunk][e];
+    }
+    u32x4_t out;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) out[e] = pack_bf16x2(t[2 * e], t[2 * e + 1]);
+    *reinterpret_cast<u32x4_t*>(p.y + (size_t)row * p.n + col) = out;
+  }
+}
+
 }  // namespace
 
 int launch_gmm_decode(hipStream_t s, const DecodeArgs& a, int nb) {
@@ -218,6 +455,38 @@ int launch_gmm_decode(hipStream_t s, const DecodeArgs& a, int nb) {
     case 128: return launch_nb<128>(s, a);
     default: return hipErrorInvalidValue;
   }
+}
+
+
+size_t gmm_rows_workspace_bytes(int m, int n, int pieces) {
+  return 256 + (size_t)m * n * sizeof(float) * (pieces > 0 ? pieces : 1);
+}
+
+int launch_gmm_rows(hipStream_t s, const DecodeArgs& a, int num_cus, void* workspace, size_t workspace_bytes) {
+  if (a.m <= 0 || a.n <= 0 || a.g <= 0) return hipSuccess;
+  if (a.n % 8 != 0 || a.n > 2048 || !workspace || (reinterpret_cast<uintptr_t>(workspace) & 15) != 0) return hipErrorInvalidValue;
+  const size_t per_piece = (size_t)a.m * a.n * sizeof(float);
+  if (workspace_bytes < 256 + per_piece) return hipErrorInvalidValue;
+  RowsGeom q;
+  q.wgs = 2 * (num_cus > 0 ? num_cus : 256);  // measured best on the decode shape: more pieces cost more in partial sums than they gain in balance
+  q.lpr = a.n / 8;
+  q.rps = kThreads / q.lpr;
+  q.max_c = (int)((workspace_bytes - 256) / per_piece < 1024 ? (workspace_bytes - 256) / per_piece : 1024);
+  q.min_rows = q.rps * kRowsDepth * 2;
+  const size_t lds = (size_t)kMaxSeg * 8 + (size_t)q.rps * kRows * a.n * sizeof(float);
+  if (lds > 64 * 1024) {
+    const int rc = (int)hipFuncSetAttribute(reinterpret_cast<const void*>(gmm_rows_kernel),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (rc != hipSuccess) return rc;
+  }
+  RowsHeader* header = static_cast<RowsHeader*>(workspace);
+  float* partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + 256);
+  hipLaunchKernelGGL(gmm_rows_kernel, dim3(q.wgs), dim3(kThreads), lds, s, a, q, header, partials);
+  int rc = (int)hipGetLastError();
+  if (rc != hipSuccess) return rc;
+  const int col_blocks = (a.n + 255) / 256;
+  hipLaunchKernelGGL(gmm_rows_finish_kernel, dim3(a.m * col_blocks), dim3(kThreads), 0, s, a, header, partials);
+  return (int)hipGetLastError();
 }
 
 }  // namespace rd

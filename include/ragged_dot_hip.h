@@ -29,6 +29,8 @@ extern "C" {
 
 enum rd_dtype { RD_DTYPE_BF16 = 0, RD_DTYPE_F32 = 1 };
 
+#define RD_DECODE_ROWS (-1) /* rd_plan.decode_nb: the streaming kernel that cuts each expert's weights into whole-row slices */
+
 enum rd_status {
   RD_OK = 0,
   RD_ERR_INVALID_ARGUMENT = -1, /* bad shape / null pointer / unknown enum */
@@ -54,7 +56,9 @@ typedef struct rd_plan {
   int variant; /* index into the variant table, or -1: let the library choose by shape */
   int group_m; /* tile walk: row tiles per L2-sharing block (tgmm: per band); 0 = default */
   int group_n; /* tile walk: column tiles per block (rd_gmm only); 0 = default */
-  int decode_nb; /* rd_gmm only: > 0 selects the skinny-m streaming kernel with this many columns per work-group */
+  int decode_nb; /* rd_gmm only, for a few rows per group: > 0 selects the streaming kernel that gives each work-group
+                    this many columns (32, 64 or 128) of one expert; RD_DECODE_ROWS the one that gives it whole rows
+                    for a slice of the contraction range (fp32 partial sums in the workspace, n <= 2048) */
   int split_k; /* rd_gmm only: 0 = when the tiles do not fill the device's last round, cut those tiles' contraction
                   range over several work-groups (fp32 partial sums in the workspace); -1 = never */
 } rd_plan;

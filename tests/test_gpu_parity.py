@@ -211,7 +211,7 @@ def test_decode_config():
     gsn = gs.cpu().numpy()
     assert int(gsn.sum()) == 64 and int((gsn > 0).sum()) == 53
     y_ref = oracle.gmm(util.to_np(x), util.to_np(A), gsn)
-    for nb in (32, 64, 128):
+    for nb in (32, 64, 128, _capi.RD_DECODE_ROWS):   # column strips of nb, or whole-row slices
         from gpu_ragged_dot_amd import ops
         y = ops._gmm_fwd(x, A, gs, 64, 64, 64, False, False, None, torch.float32, 512, plan=_capi.Plan(-1, 0, nb))
         util.assert_close_rows(util.to_np(y), y_ref, 64, util.BF16_EPS, f"decode nb={nb}")
@@ -226,7 +226,7 @@ def test_decode_kernel_long_groups_and_tail():
     lhs, rhs, _, _, _ = util.make_case(5, m, k, n, g, 1.0, True, scale_rhs=True)
     gs = np.array([0, 11, 1, 0, 9, 5], np.int32)  # sum 26 < 40
     from gpu_ragged_dot_amd import ops
-    for nb in (32, 64, 128):
+    for nb in (32, 64, 128, _capi.RD_DECODE_ROWS):
         y = ops._gmm_fwd(util.bf16_dev(lhs), util.bf16_dev(rhs), torch.from_numpy(gs), 64, 64, 64, False, False, None,
                          torch.float32, 512, plan=_capi.Plan(-1, 0, nb))
         y = util.to_np(y)

@@ -117,7 +117,7 @@ def test_planner_choices():
     p = planner.select_plan(_capi.OP_TGMM, 171, 58, 77, 8, dtype=_capi.RD_DTYPE_F32)
     assert vs[p.variant].dtype == _capi.RD_DTYPE_F32
     p = planner.select_plan(_capi.OP_GMM, 64, 2048, 768, 128)
-    assert p.decode_nb > 0  # a few rows per expert -> streaming kernel
+    assert p.decode_nb == _capi.RD_DECODE_ROWS  # a few rows per expert -> streaming kernel (whole-row slices)
     p = planner.select_plan(_capi.OP_GMM_TRANS, 64, 2048, 768, 128)
     assert p.decode_nb == 0
     p = planner.select_plan(_capi.OP_GMM, 16384, 4096, 14336, 8)
