@@ -450,12 +450,14 @@ __device__ __forceinline__ void gemm_tile_pingpong(const bf16_bits* __restrict__
     const unsigned char* ra = smem + (kt % C::STAGES) * C::STAGE_BYTES;
     const unsigned char* rb = ra + C::A_BYTES;
     bf16x8_t fa[C::KSTEPS][C::TM], fb[C::KSTEPS][C::TN];
+    if (patch_live) {  // a wave without matrix-core work leaves the LDS bandwidth, which paces the loop, to the others
 #pragma unroll
-    for (int ks = 0; ks < C::KSTEPS; ++ks) {
+      for (int ks = 0; ks < C::KSTEPS; ++ks) {
 #pragma unroll
-      for (int i = 0; i < C::TM; ++i) fa[ks][i] = fra.read(ra, i, ks);
+        for (int i = 0; i < C::TM; ++i) fa[ks][i] = fra.read(ra, i, ks);
 #pragma unroll
-      for (int j = 0; j < C::TN; ++j) fb[ks][j] = frb.read(rb, j, ks);
+        for (int j = 0; j < C::TN; ++j) fb[ks][j] = frb.read(rb, j, ks);
+      }
     }
     // The slot of slab kt-1 is free: both groups finished reading it before the barrier that opened this phase.
     if (kt + C::STAGES - 1 < nk) issue_slab(kt + C::STAGES - 1);

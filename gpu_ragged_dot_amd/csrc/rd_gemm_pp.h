@@ -167,12 +167,14 @@ __device__ __forceinline__ void gemm_tile_pingpong_mixed(const bf16_bits* __rest
     if (do_a) issue_a(qa + C::A_S - 1);
     if (do_b) issue_b(qb + C::B_S - 1);
     __builtin_amdgcn_sched_barrier(0);
+    if (patch_live) {  // a wave without matrix-core work leaves the LDS bandwidth, which paces the loop, to the others
 #pragma unroll
-    for (int ks = 0; ks < C::KSTEPS; ++ks) {
+      for (int ks = 0; ks < C::KSTEPS; ++ks) {
 #pragma unroll
-      for (int i = 0; i < C::TM; ++i) fa[ks][i] = fra.read(ra, i, ks + KA);
+        for (int i = 0; i < C::TM; ++i) fa[ks][i] = fra.read(ra, i, ks + KA);
 #pragma unroll
-      for (int j = 0; j < C::TN; ++j) fb[ks][j] = frb.read(rb, j, ks + KB);
+        for (int j = 0; j < C::TN; ++j) fb[ks][j] = frb.read(rb, j, ks + KB);
+      }
     }
     // Own share of everything the next phase reads has landed.  The immediate count is exact in the steady state;
     // near the end, where fewer loads are in flight than it assumes, wait for all of them.
