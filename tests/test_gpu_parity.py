@@ -234,6 +234,27 @@ def test_decode_kernel_long_groups_and_tail():
         assert not np.any(y[26:])
 
 
+@pytest.mark.parametrize("g,active,rows_each", [(600, 40, 1), (1500, 1500, 1), (300, 299, 2), (257, 3, 7)],
+                         ids=["g600-sparse", "g1500-all-active", "g300-two-rows", "g257-few-long"])
+def test_decode_rows_kernel_many_groups(g, active, rows_each):
+    """The whole-row streaming kernel with more groups than one scan slab holds (256), and with more non-empty groups
+    than it launches work-groups (each work-group then serves several experts in turn)."""
+    from gpu_ragged_dot_amd import ops
+    print(f"decode rows kernel g={g} active={active} rows_each={rows_each}", flush=True)
+    rng = np.random.default_rng(g)
+    k, n = 136, 72
+    gs = np.zeros(g, np.int32)
+    gs[rng.choice(g, active, replace=False)] = rows_each
+    m = int(gs.sum()) + 5
+    lhs = oracle.round_to(rng.standard_normal((m, k)).astype(np.float32), "bfloat16")
+    rhs = oracle.round_to((rng.standard_normal((g, k, n)) / k ** 0.5).astype(np.float32), "bfloat16")
+    y = ops._gmm_fwd(util.bf16_dev(lhs), util.bf16_dev(rhs), torch.from_numpy(gs), 64, 64, 64, False, False, None,
+                     torch.float32, 512, plan=_capi.Plan(-1, 0, _capi.RD_DECODE_ROWS))
+    y = util.to_np(y)
+    util.assert_close_rows(y, oracle.gmm(lhs, rhs, gs), int(gs.sum()), util.BF16_EPS, "rows kernel")
+    assert not np.any(y[int(gs.sum()):])
+
+
 # ---------------------------------------------------------------------------------------------------------------------
 # what the reference leaves undefined or never checks
 # ---------------------------------------------------------------------------------------------------------------------
