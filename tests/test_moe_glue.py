@@ -118,7 +118,9 @@ def test_oracle_dispatch_combine_adjoint_and_definition():
 # ---------------------------------------------------------------------------------------------------------------------
 
 ROUTE_CASES = [(0, 1, 1, 1, 0), (1, 7, 2, 3, 0), (2, 40, 3, 5, 0.2), (3, 8, 8, 128, 0), (4, 33, 4, 2, 0.5),
-               (6, 4096, 8, 256, 0.0), (7, 5000, 2, 8, 0.05), (8, 3000, 6, 1500, 0.1), (9, 1030, 1, 12288, 0.0)]
+               (6, 4096, 8, 256, 0.0), (7, 5000, 2, 8, 0.05), (8, 3000, 6, 1500, 0.1), (9, 1030, 1, 12288, 0.0),
+               (10, 250000, 2, 12288, 0.01),   # per-chunk histograms would pass 4M entries: the chunk length doubles
+               (11, 2000, 64, 32, 0.0)]       # the largest top_k
 
 
 @pytest.mark.gpu
