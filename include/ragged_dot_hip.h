@@ -51,7 +51,7 @@ typedef struct rd_variant_info {
   char name[48];
 } rd_variant_info;
 
-/* Launch plan for one call; the host planner (or the caller) fills it.  Zero-initialised = library defaults. */
+/* Launch plan for one call; the host planner (or the caller) fills it.  variant = -1 with every other field 0 = library defaults. */
 typedef struct rd_plan {
   int variant; /* index into the variant table, or -1: let the library choose by shape */
   int group_m; /* tile walk: row tiles per L2-sharing block (tgmm: per band); 0 = default */
