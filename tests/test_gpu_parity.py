@@ -405,6 +405,37 @@ def test_float32_trans_ragged_dot(c):
     assert not np.any(util.to_np(out)[gs == 0])
 
 
+@pytest.mark.parametrize("shape", [(1030, 264, 392, 5), (515, 99, 131, 3), (600, 130, 262, 4), (2048, 128, 256, 2)],
+                         ids=lambda s: "m%d_k%d_n%d_g%d" % s)
+def test_float32_every_tile_shape(shape):
+    """Each compiled float32 tile shape, forced through the plan, on shapes that take the 16-byte loads (all of k, n
+    multiples of 4), the element loads (odd k, n) and a mix (k multiple of 2 only), against a float64 contraction."""
+    from gpu_ragged_dot_amd import ops
+    m, k, n, g = shape
+    print("f32 tiles", shape, flush=True)
+    rng = np.random.default_rng(m + k + n)
+    lhs, rhs, dout = (rng.normal(size=s).astype(np.float32) for s in ((m, k), (g, k, n), (m, n)))
+    gs = oracle.generate_group_sizes(11 + m, g, m - 37)
+    rows = np.arange(m) < m - 37
+    f64 = dict(out_dtype="float32", acc=np.float64)
+    o_ref = oracle.gmm(lhs, rhs, gs, **f64)
+    dlhs_ref = oracle.gmm(dout, rhs, gs, trans_rhs=True, **f64)
+    drhs_ref = oracle.tgmm(lhs, dout, gs, **f64)
+    x_t, A_t, d_t, gs_t = (torch.from_numpy(a).cuda() for a in (lhs, rhs, dout, gs))
+    ids = [i for i, v in enumerate(_capi.variants()) if v.dtype == _capi.RD_DTYPE_F32]
+    assert len(ids) >= 2
+    for vid in ids:
+        hp = (64, 64, 64)
+        o = ops._gmm_fwd(x_t, A_t, gs_t, *hp, False, False, None, torch.float32, 512, plan=_capi.Plan(vid))
+        dl = ops._gmm_fwd(d_t, A_t, gs_t, *hp, True, False, None, torch.float32, 512, plan=_capi.Plan(vid))
+        dr = ops._tgmm_fwd(x_t, d_t, gs_t, *hp, False, None, torch.float32, 512, plan=_capi.Plan(vid))
+        assert float(np.max(oracle.err_fn(util.to_np(o), o_ref, mask=rows))) < F32_EPS
+        assert float(np.max(oracle.err_fn(util.to_np(dl), dlhs_ref, mask=rows))) < F32_EPS
+        assert float(np.max(oracle.err_fn(util.to_np(dr), drhs_ref, axis=(-1, -2), mask=gs != 0))) < F32_TGMM_EPS
+        assert not np.any(util.to_np(o)[m - 37:]) and not np.any(util.to_np(dl)[m - 37:])
+        assert not np.any(util.to_np(dr)[gs == 0])
+
+
 # ---------------------------------------------------------------------------------------------------------------------
 # HIP graph capture: no entry point reads device data on the host, so a captured step replays correctly
 # ---------------------------------------------------------------------------------------------------------------------
