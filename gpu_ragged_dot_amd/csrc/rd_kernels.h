@@ -3,6 +3,7 @@
 #pragma once
 #include "rd_gemm_dlds.h"
 #include "rd_gemm_f32.h"
+#include "rd_gemm_w4.h"
 #include "rd_gemm_pp.h"
 #include "rd_gemm_tile.h"
 
@@ -45,11 +46,17 @@ struct TgmmArgs {
 // A value every lane holds identically, moved to a scalar register.
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
+template <class C, class = void>
+struct IsW4 { static constexpr bool value = false; };
+template <class C>
+struct IsW4<C, decltype((void)C::W4)> { static constexpr bool value = true; };
+
 template <class C>
 __device__ __forceinline__ void run_tile(const typename C::Elem* Ap, int lda, int a_lim, const typename C::Elem* Bp,
                                          int ldb, int b_lim, int klen, typename C::Elem* Op, int ldo,
                                          typename C::Elem* smem, const SplitK& sk = SplitK()) {
   if constexpr (C::F32) gemm_tile_f32<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
+  else if constexpr (IsW4<C>::value) gemm_tile_w4<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
   else if constexpr (C::MIXED) gemm_tile_pingpong_mixed<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
   else if constexpr (C::DLDS && C::PINGPONG) gemm_tile_pingpong<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
   else if constexpr (C::DLDS) gemm_tile_dlds<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);

@@ -27,6 +27,10 @@ namespace rd {
 typedef F32Cfg<RD_BM, RD_BN, /*A K-major*/ true, /*B K-major*/ false> CfgNN;
 typedef F32Cfg<RD_BM, RD_BN, true, true> CfgNT;
 typedef F32Cfg<RD_BM, RD_BN, false, false> CfgTN;
+#elif RD_DLDS == 3
+typedef W4Cfg<RD_BM, RD_BN, /*A K-major*/ true, /*B K-major*/ false, RD_STAGES> CfgNN;
+typedef W4Cfg<RD_BM, RD_BN, true, true, RD_STAGES> CfgNT;
+typedef W4Cfg<RD_BM, RD_BN, false, false, RD_STAGES> CfgTN;
 #elif RD_DLDS == 2
 // one LDS ring per operand: K-major A in 64-wide slabs (3 slots), everything else in 32-wide slabs (4 slots)
 typedef PpCfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, /*A K-major*/ true, /*B K-major*/ false, 64, 3, 32, 4> CfgNN;
