@@ -32,9 +32,11 @@ typedef W4Cfg<RD_BM, RD_BN, /*A K-major*/ true, /*B K-major*/ false, RD_STAGES> 
 typedef W4Cfg<RD_BM, RD_BN, true, true, RD_STAGES> CfgNT;
 typedef W4Cfg<RD_BM, RD_BN, false, false, RD_STAGES> CfgTN;
 #elif RD_DLDS == 2
-// one LDS ring per operand: K-major A in 64-wide slabs (3 slots), everything else in 32-wide slabs (4 slots)
+// one LDS ring per operand: one K-major operand in 64-wide slabs (3 slots) - the activations in the forward product,
+// the weights A[g,n,k] with trans_rhs (measured 1-3 % ahead of giving them to dout) - everything else in 32-wide
+// slabs (4 slots)
 typedef PpCfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, /*A K-major*/ true, /*B K-major*/ false, 64, 3, 32, 4> CfgNN;
-typedef PpCfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, true, true, 64, 3, 32, 4> CfgNT;
+typedef PpCfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, true, true, 32, 4, 64, 3> CfgNT;
 typedef PpCfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, false, false, 32, 4, 32, 4> CfgTN;
 #elif RD_DLDS
 typedef DldsCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, /*A K-major*/ true, /*B K-major*/ false, RD_STAGES, RD_PINGPONG != 0> CfgNN;
