@@ -126,6 +126,24 @@ def test_planner_choices():
     assert (vs[p.variant].tile_m, vs[p.variant].tile_n) == (128, 128)  # explicit request -> nearest compiled shape
 
 
+def test_default_plan_scales_the_tile_with_the_problem():
+    """The library's shape-only default (no tuned-table entry): 256 x 256 cores for many rounds of tiles or a long
+    contraction, the 128-row cores when those would leave compute units idle, register-staged tiles for small outputs;
+    all three products; float32 picks its larger tile only when the output fills the device with it."""
+    vs = {v.id: v for v in _capi.variants()}
+    tile = lambda op, m, k, n, g, **kw: (lambda v: (v.tile_m, v.tile_n))(vs[_capi.default_plan(op, m, k, n, g, **kw).variant])
+    for op in (_capi.OP_GMM, _capi.OP_GMM_TRANS, _capi.OP_TGMM):
+        assert tile(op, 16384, 4096, 14336, 8) == (256, 256)
+        assert tile(op, 32768, 7168, 2048, 256) == (256, 256)
+    assert tile(_capi.OP_GMM, 6144, 6144, 1536, 6) == (256, 256)      # few tiles, long contraction
+    assert tile(_capi.OP_GMM, 16384, 2048, 2048, 8) == (128, 256)     # two rounds of 256-tiles: the 128-row core fills the device better
+    assert tile(_capi.OP_GMM_TRANS, 8192, 4096, 256, 16) == (128, 128)
+    assert tile(_capi.OP_TGMM, 4096, 1024, 1024, 8) == (128, 128)
+    assert max(tile(_capi.OP_GMM, 2048, 4096, 512, 4)) <= 128 and max(tile(_capi.OP_GMM, 256, 64, 64, 4)) <= 128
+    assert tile(_capi.OP_GMM, 8192, 4096, 4096, 8, dtype=_capi.RD_DTYPE_F32) == (128, 128)
+    assert tile(_capi.OP_GMM, 512, 256, 256, 4, dtype=_capi.RD_DTYPE_F32) == (64, 64)
+
+
 def test_cpu_tensors_are_rejected_loudly():
     import gpu_ragged_dot_amd as rd
 
