@@ -181,31 +181,43 @@ struct SplitK {
 
 // Returns true when the caller holds the complete sums and must store them.  All threads of the work-group call it,
 // after the last barrier of the K loop (it uses the first bytes of LDS to broadcast the arrival index).
+//
+// The pieces of a tile run on different XCDs, whose L2 caches do not see each other's lines.  A device-scope fence would
+// make them agree by writing back and invalidating a whole L2 - tens of microseconds each, one after the other, for
+// every piece - so the partial sums go around the problem instead: they are stored and loaded with the sc1 cache policy
+// (coherent at device scope: written through, re-fetched), and the only ordering needed is that a piece's stores have
+// completed before its arrival is counted.
+constexpr int kCachePolicyDevice = 16;  // sc1 in the aux operand of the buffer intrinsics
+
 template <class C>
 __device__ __forceinline__ bool splitk_combine(f32x16_t (&acc)[C::TM][C::TN], const SplitK& sk, int tid,
                                                unsigned char* smem) {
   if (sk.parts <= 1) return true;
-  constexpr int QUADS = C::TM * C::TN * 4;  // float4 per thread
-  f32x4_t* mine = reinterpret_cast<f32x4_t*>(sk.partials) + (size_t)sk.part * (QUADS * C::NT) + tid;
+  constexpr int QUADS = C::TM * C::TN * 4;             // 16-byte vectors per thread
+  constexpr int PIECE_BYTES = QUADS * C::NT * 16;      // one piece's accumulators
+  __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)sk.partials, 0, sk.parts * PIECE_BYTES, kBufferFlags);
+  const int lane_off = tid * 16;
 #pragma unroll
   for (int i = 0; i < C::TM; ++i)
 #pragma unroll
     for (int j = 0; j < C::TN; ++j)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        f32x4_t v;
-        v[0] = acc[i][j][4 * g + 0]; v[1] = acc[i][j][4 * g + 1]; v[2] = acc[i][j][4 * g + 2]; v[3] = acc[i][j][4 * g + 3];
-        mine[((i * C::TN + j) * 4 + g) * C::NT] = v;
+        // whole-vector casts only: a bit cast of a single vector element reads element 0 whatever the index
+        f32x4_t q;
+        q[0] = acc[i][j][4 * g + 0]; q[1] = acc[i][j][4 * g + 1]; q[2] = acc[i][j][4 * g + 2]; q[3] = acc[i][j][4 * g + 3];
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, q), rsrc, lane_off + ((i * C::TN + j) * 4 + g) * (C::NT * 16),
+                                                   sk.part * PIECE_BYTES, kCachePolicyDevice);
       }
-  __threadfence();  // the partial sums are visible device-wide before the arrival is
-  __syncthreads();
+  wait_vmcnt<0>();   // this thread's stores have completed (a work-group-scope fence would not wait for them)
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();   // ... and every thread's
   int32_t* slot = reinterpret_cast<int32_t*>(smem);
-  if (tid == 0) *slot = atomicAdd(sk.counter, 1);
+  if (tid == 0) *slot = __hip_atomic_fetch_add(sk.counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   const int arrived = *slot;
   __syncthreads();  // everyone has read the slot before the epilogue reuses LDS
   if (arrived != sk.parts - 1) return false;
-  __threadfence();  // see the other pieces' stores, not stale cache lines
   // Sum the pieces in index order, this work-group's own included, so that the result does not depend on which piece
   // happened to arrive last.
 #pragma unroll
@@ -215,14 +227,15 @@ __device__ __forceinline__ bool splitk_combine(f32x16_t (&acc)[C::TM][C::TN], co
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
   for (int s = 0; s < sk.parts; ++s) {
-    const f32x4_t* other = reinterpret_cast<const f32x4_t*>(sk.partials) + (size_t)s * (QUADS * C::NT) + tid;
 #pragma unroll
     for (int i = 0; i < C::TM; ++i)
 #pragma unroll
       for (int j = 0; j < C::TN; ++j)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          const f32x4_t v = other[((i * C::TN + j) * 4 + g) * C::NT];
+          const u32x4_t raw = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + ((i * C::TN + j) * 4 + g) * (C::NT * 16),
+                                                                        s * PIECE_BYTES, kCachePolicyDevice);
+          const f32x4_t v = __builtin_bit_cast(f32x4_t, raw);
           acc[i][j][4 * g + 0] += v[0]; acc[i][j][4 * g + 1] += v[1]; acc[i][j][4 * g + 2] += v[2]; acc[i][j][4 * g + 3] += v[3];
         }
   }

@@ -27,6 +27,7 @@ struct GmmArgs {
   float* partials;     // [split_slots][BM * BN] fp32
   int32_t* counters;   // [split_slots], zero at launch
   int split_slots;     // work-groups appended to the launch for the split pieces
+  int max_parts;       // > 0: most pieces a tile is cut into, as the caller asked; 0: chosen from k
   int num_cus;         // tiles the device runs at a time (one work-group per compute unit)
   int main_grid;       // launch indices below this walk whole tiles (set by the launcher)
 };
@@ -74,14 +75,26 @@ struct SplitPlan {
 constexpr int kMaxSplitParts = 8;
 constexpr int kMinSplitK = 512;  // contraction elements a piece must keep
 
-__device__ __forceinline__ SplitPlan split_plan(int total, int n_tiles, int k, int slots, int num_cus) {
+__device__ __forceinline__ SplitPlan split_plan(int total, int n_tiles, int k, int slots, int num_cus, int max_parts) {
   SplitPlan sp{total, 1, 0};
   if (slots <= 0 || total <= 0) return sp;
   const int live = total * n_tiles;
   const int first = ((live / num_cus) * num_cus) / n_tiles;
   const int tiles = (total - first) * n_tiles;
   if (tiles <= 0) return sp;
+  // The piece that arrives last reads every piece's 256 KB of partial sums at what one compute unit can pull (about
+  // 25 GB/s: ~10 us per piece), so the gain of a finer cut, T/parts for a K loop of T us, is soon eaten: parts ~
+  // sqrt(T / 10 us), with T ~ k / 32 x 0.77 us, i.e. sqrt(k) / 20 - and below k = 6400 (4 pieces) cutting was measured
+  // to gain nothing.  max_parts > 0 is the caller's own choice and is taken as it is.
   int parts = imin(imin(slots / tiles, kMaxSplitParts), k / kMinSplitK);
+  if (max_parts > 0) {
+    parts = imin(parts, max_parts);
+  } else {
+    int by_k = 1;
+    while ((by_k + 1) * (by_k + 1) * 400 <= k) ++by_k;
+    if (by_k < 4) return sp;
+    parts = imin(parts, by_k);
+  }
   if (parts < 2) return sp;
   sp.first_row = first; sp.parts = parts; sp.tiles = tiles;
   return sp;
@@ -113,7 +126,7 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
   // Everything read through the map is the same for the whole work-group: pin it to scalar registers.
   const int total = imin(uniform(*p.total_tiles), p.U);
   SplitPlan sp{total, 1, 0};
-  if constexpr (C::SPLITK) sp = split_plan(total, p.n_tiles, p.k, p.split_slots, p.num_cus);
+  if constexpr (C::SPLITK) sp = split_plan(total, p.n_tiles, p.k, p.split_slots, p.num_cus, p.max_parts);
 
   int mi, nj;
   SplitK sk;

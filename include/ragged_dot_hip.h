@@ -59,8 +59,9 @@ typedef struct rd_plan {
   int decode_nb; /* rd_gmm only, for a few rows per group: > 0 selects the streaming kernel that gives each work-group
                     this many columns (32, 64 or 128) of one expert; RD_DECODE_ROWS the one that gives it whole rows
                     for a slice of the contraction range (fp32 partial sums in the workspace, n <= 2048) */
-  int split_k; /* rd_gmm only: 0 = when the tiles do not fill the device's last round, cut those tiles' contraction
-                  range over several work-groups (fp32 partial sums in the workspace); -1 = never */
+  int split_k; /* rd_gmm only: 0 = when the tiles do not fill the device's last round and k >= 6400, cut those tiles'
+                  contraction range over up to sqrt(k)/20 work-groups (fp32 partial sums in the workspace); n > 0 =
+                  cut them over up to n (at most 8) whatever k is; -1 = never */
 } rd_plan;
 
 int rd_abi_version(void);

@@ -165,7 +165,7 @@ def test_k_split_of_last_round(vid, vname, shape, trans_rhs):
     x = util.bf16_dev(lhs)
     A = util.bf16_dev(np.ascontiguousarray(np.swapaxes(rhs, 1, 2)) if trans_rhs else rhs)
     gs_d = torch.from_numpy(gs).cuda()
-    split, whole = _capi.Plan(vid, 2, 0, 2, split_k=0), _capi.Plan(vid, 2, 0, 2, split_k=-1)
+    split, whole = _capi.Plan(vid, 2, 0, 2, split_k=8), _capi.Plan(vid, 2, 0, 2, split_k=-1)  # 8: cut whatever k is
     need = _capi.lib.rd_gmm_workspace_bytes(m, g, ctypes.byref(split))
     assert need > _capi.lib.rd_gmm_workspace_bytes(m, g, ctypes.byref(whole))
     ws = torch.empty(need, dtype=torch.uint8, device="cuda")

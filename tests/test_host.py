@@ -136,7 +136,7 @@ def test_default_plan_scales_the_tile_with_the_problem():
         assert tile(op, 16384, 4096, 14336, 8) == (256, 256)
         assert tile(op, 32768, 7168, 2048, 256) == (256, 256)
     assert tile(_capi.OP_GMM, 6144, 6144, 1536, 6) == (256, 256)      # few tiles, long contraction
-    assert tile(_capi.OP_GMM, 16384, 2048, 2048, 8) == (128, 256)     # two rounds of 256-tiles: the 128-row core fills the device better
+    assert tile(_capi.OP_GMM, 65536, 512, 512, 64) == (128, 256)      # short contraction: two work-groups per compute unit hide the tile set-up
     assert tile(_capi.OP_GMM_TRANS, 8192, 4096, 256, 16) == (128, 128)
     assert tile(_capi.OP_TGMM, 4096, 1024, 1024, 8) == (128, 128)
     assert max(tile(_capi.OP_GMM, 2048, 4096, 512, 4)) <= 128 and max(tile(_capi.OP_GMM, 256, 64, 64, 4)) <= 128
