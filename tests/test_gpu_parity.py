@@ -187,6 +187,16 @@ def test_k_split_of_last_round(vid, vname, shape, trans_rhs):
     assert np.array_equal(outs[0], outs[1])
     scale = np.abs(y_ref).max()
     assert np.abs(outs[0].astype(np.float32) - outs[2].astype(np.float32)).max() <= 2 ** -7 * scale
+    # Same workspace, other data: no piece may see a partial sum of the call before (the pieces of a tile run on
+    # different XCDs, whose L2 caches hold what the previous call read).  Scaling by -2 is exact in bf16 and fp32.
+    x2 = (x.float() * -2.0).to(torch.bfloat16)
+    y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    rc = _capi.lib.rd_gmm(torch.cuda.current_stream().cuda_stream, x2.data_ptr(), A.data_ptr(), gs_d.data_ptr(),
+                          y.data_ptr(), m, k, n, g, int(trans_rhs), _capi.RD_DTYPE_BF16, ctypes.byref(split),
+                          ws.data_ptr(), ws.numel())
+    torch.cuda.synchronize()
+    assert rc == 0, _capi.lib.rd_last_error()
+    assert np.array_equal(util.to_np(y).astype(np.float32), -2.0 * outs[0].astype(np.float32))
 
 
 # ---------------------------------------------------------------------------------------------------------------------
