@@ -13,12 +13,6 @@
 #pragma once
 #include "rd_common.h"
 
-// Hook for timing experiments: a build may define RD_MARK(id) to record a timestamp at each pipeline phase.
-#ifndef RD_MARK
-#define RD_MARK(id)
-#define RD_MARK_DECL
-#endif
-
 namespace rd {
 
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, bool A_KMAJOR_, bool B_KMAJOR_, int STAGES_,
@@ -283,7 +277,6 @@ __device__ __forceinline__ void gemm_tile_dlds(const bf16_bits* __restrict__ Ap,
                                                const bf16_bits* __restrict__ Bp, int ldb, int b_lim, int klen,
                                                bf16_bits* __restrict__ Op, int ldo, bf16_bits* smem_,
                                                const SplitK& sk = SplitK()) {
-  RD_MARK_DECL;
   unsigned char* smem = reinterpret_cast<unsigned char*>(smem_);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -337,13 +330,10 @@ __device__ __forceinline__ void gemm_tile_dlds(const bf16_bits* __restrict__ Ap,
     if (s < nk) { issue_loads(s, 0, L); la.advance(); lb.advance(); }
 
   for (int kt = 0; kt < nk; ++kt) {
-    RD_MARK(0);
     // Slab kt must have landed; the STAGES-2 younger ones may still be in flight.  Near the end fewer loads were
     // issued after slab kt than that, so wait for everything.
     if (kt + C::STAGES - 2 < nk) wait_vmcnt<(C::STAGES - 2) * L>(); else wait_vmcnt<0>();
-    RD_MARK(1);
     __builtin_amdgcn_s_barrier();  // every wave's part of slab kt is in LDS, and slab kt-1 is no longer being read
-    RD_MARK(2);
     const bool more = kt + C::STAGES - 1 < nk;
 
     const unsigned char* ra = smem + (kt % C::STAGES) * C::STAGE_BYTES;
@@ -383,7 +373,6 @@ __device__ __forceinline__ void gemm_tile_dlds(const bf16_bits* __restrict__ Ap,
       __builtin_amdgcn_sched_barrier(0);
     }
     if (more) { la.advance(); lb.advance(); }
-    RD_MARK(3);
   }
 
   __builtin_amdgcn_s_barrier();  // the ring is no longer read by any wave

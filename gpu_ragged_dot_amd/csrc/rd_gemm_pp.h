@@ -79,7 +79,6 @@ __device__ __forceinline__ void gemm_tile_pingpong_mixed(const bf16_bits* __rest
                                                          const bf16_bits* __restrict__ Bp, int ldb, int b_lim,
                                                          int klen, bf16_bits* __restrict__ Op, int ldo,
                                                          bf16_bits* smem_, const SplitK& sk = SplitK()) {
-  RD_MARK_DECL;
   unsigned char* smem = reinterpret_cast<unsigned char*>(smem_);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -181,9 +180,7 @@ __device__ __forceinline__ void gemm_tile_pingpong_mixed(const bf16_bits* __rest
     if (steady) wait_vmcnt<Cnt::allowed(PAR)>(); else wait_vmcnt<0>();
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
     __builtin_amdgcn_sched_barrier(0);
-    RD_MARK(0);
     __builtin_amdgcn_s_barrier();
-    RD_MARK(1);
     __builtin_amdgcn_sched_barrier(0);
     // ---- compute phase --------------------------------------------------------------------------------------------
     __builtin_amdgcn_s_setprio(1);
@@ -198,9 +195,7 @@ __device__ __forceinline__ void gemm_tile_pingpong_mixed(const bf16_bits* __rest
     }
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);
-    RD_MARK(2);
     __builtin_amdgcn_s_barrier();
-    RD_MARK(3);
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -209,11 +204,9 @@ __device__ __forceinline__ void gemm_tile_pingpong_mixed(const bf16_bits* __rest
     if (p + 1 < nk) phase(p + 1, pp_detail::Parity<1>{});
   }
   if (group == 0) __builtin_amdgcn_s_barrier();
-  RD_MARK(4);
 
   if (!splitk_combine<C>(acc, sk, tid, smem)) return;
   store_accumulators<C>(acc, wm, wn, wave, lane, a_lim, b_lim, Op, ldo, smem);
-  RD_MARK(5);
 }
 
 }  // namespace rd
