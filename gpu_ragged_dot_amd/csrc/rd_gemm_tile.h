@@ -17,9 +17,14 @@
 
 namespace rd {
 
-template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, bool A_KMAJOR_, bool B_KMAJOR_, bool VEC_>
+// Src: element type of the operands and the output in HBM.  bf16_bits: bf16 in, bf16 out.  float: float32 arrays whose
+// elements are rounded to bf16 (nearest even) on their way into LDS, multiplied on the bf16 matrix cores with fp32
+// accumulation and stored as float32 - the reference's compute_dtype = bfloat16 on float32 arrays
+// (gpu_ragged_dot.py:116-119, 145, 149).
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, bool A_KMAJOR_, bool B_KMAJOR_, bool VEC_,
+          typename Src = bf16_bits>
 struct TileCfg {
-  typedef bf16_bits Elem;
+  typedef Src Elem;
   static constexpr bool F32 = false;
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
   static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = VEC_, DLDS = false, PINGPONG = false, MIXED = false,
@@ -44,7 +49,7 @@ struct TileCfg {
 };
 
 // Moves one operand's [T x BK] slab HBM -> registers -> LDS in 16-byte chunks, NT threads cooperating.
-template <int T, int BK, int NT, bool KMAJOR, int STRIDE, bool VEC>
+template <int T, int BK, int NT, bool KMAJOR, int STRIDE, bool VEC, typename Src = bf16_bits>
 struct OperandStager {
   static constexpr int CPR = KMAJOR ? BK / 8 : T / 8;  // 16-byte chunks per LDS row
   static constexpr int ROWS = KMAJOR ? T : BK;
@@ -53,11 +58,24 @@ struct OperandStager {
   static constexpr int ROW_STEP = NT / CPR;     // LDS rows between two chunks of one thread
   static_assert(NCHUNK % NT == 0 && NT % CPR == 0 && PER >= 1, "tile too small for this many threads");
 
-  const bf16_bits* base;  // tile origin in HBM
+  const Src* base;  // tile origin in HBM
   int ld, lim, klen, c, r0;
   int off[PER];  // K-major: element offset of each chunk's (clamped) row; MN-major: row * ld
 
-  __device__ __forceinline__ void init(const bf16_bits* p, int ld_, int lim_, int klen_, int tid) {
+  // 8 consecutive elements at p as one 16-byte chunk of bf16 (VEC: p is 16-byte aligned)
+  static __device__ __forceinline__ u32x4_t chunk8(const Src* p) {
+    if constexpr (sizeof(Src) == 2) {
+      return *reinterpret_cast<const u32x4_t*>(p);
+    } else {
+      const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(p), hi = *reinterpret_cast<const f32x4_t*>(p + 4);
+      return u32x4_t{pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]), pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3])};
+    }
+  }
+  static __device__ __forceinline__ bf16_bits elem(const Src* p) {
+    if constexpr (sizeof(Src) == 2) return *p; else return f32_to_bf16(*p);
+  }
+
+  __device__ __forceinline__ void init(const Src* p, int ld_, int lim_, int klen_, int tid) {
     base = p; ld = ld_; lim = lim_; klen = klen_;
     c = tid % CPR; r0 = tid / CPR;
 #pragma unroll
@@ -75,10 +93,10 @@ struct OperandStager {
       if (VEC) {
         if (KMAJOR) {
           const bool ok = !PRED || (k0 + c * 8 < klen);
-          r[i] = ok ? *reinterpret_cast<const u32x4_t*>(base + off[i] + k0) : u32x4_t{0, 0, 0, 0};
+          r[i] = ok ? chunk8(base + off[i] + k0) : u32x4_t{0, 0, 0, 0};
         } else {
           const bool ok = !PRED || (k0 + r0 + i * ROW_STEP < klen);
-          r[i] = ok ? *reinterpret_cast<const u32x4_t*>(base + (size_t)k0 * ld + off[i]) : u32x4_t{0, 0, 0, 0};
+          r[i] = ok ? chunk8(base + (size_t)k0 * ld + off[i]) : u32x4_t{0, 0, 0, 0};
         }
       } else {
         // element-granular path for pitches that are not a multiple of 16 bytes
@@ -88,10 +106,10 @@ struct OperandStager {
           bf16_bits v = 0;
           if (KMAJOR) {
             const int kk = k0 + c * 8 + e;
-            if (kk < klen) v = base[off[i] + k0 + e];
+            if (kk < klen) v = elem(base + off[i] + k0 + e);
           } else {
             const int kk = k0 + r0 + i * ROW_STEP;
-            if (kk < klen && c * 8 + e < lim) v = base[(size_t)k0 * ld + off[i] + e];
+            if (kk < klen && c * 8 + e < lim) v = elem(base + (size_t)k0 * ld + off[i] + e);
           }
           w[e >> 1] |= (uint32_t)v << ((e & 1) * 16);
         }
@@ -129,16 +147,17 @@ __device__ __forceinline__ bf16x8_t read_fragment(const bf16_bits* lds, int idx0
   }
 }
 
-// C[i, j] (i < a_lim, j < b_lim) -> Op[i*ldo + j] as bf16.  `smem` must hold C::LDS_BYTES.
+// C[i, j] (i < a_lim, j < b_lim) -> Op[i*ldo + j] in the element type of the configuration.  `smem` must hold
+// C::LDS_BYTES.
 template <class C>
-__device__ __forceinline__ void gemm_tile(const bf16_bits* __restrict__ Ap, int lda, int a_lim,
-                                          const bf16_bits* __restrict__ Bp, int ldb, int b_lim, int klen,
-                                          bf16_bits* __restrict__ Op, int ldo, bf16_bits* smem) {
+__device__ __forceinline__ void gemm_tile(const typename C::Elem* __restrict__ Ap, int lda, int a_lim,
+                                          const typename C::Elem* __restrict__ Bp, int ldb, int b_lim, int klen,
+                                          typename C::Elem* __restrict__ Op, int ldo, bf16_bits* smem) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;
 
-  typedef OperandStager<C::BM, C::BK, C::NT, C::A_KMAJOR, C::A_STRIDE, C::VEC> StA;
-  typedef OperandStager<C::BN, C::BK, C::NT, C::B_KMAJOR, C::B_STRIDE, C::VEC> StB;
+  typedef OperandStager<C::BM, C::BK, C::NT, C::A_KMAJOR, C::A_STRIDE, C::VEC, typename C::Elem> StA;
+  typedef OperandStager<C::BN, C::BK, C::NT, C::B_KMAJOR, C::B_STRIDE, C::VEC, typename C::Elem> StB;
   StA sa; StB sb;
   sa.init(Ap, lda, a_lim, klen, tid);
   sb.init(Bp, ldb, b_lim, klen, tid);
@@ -204,7 +223,10 @@ __device__ __forceinline__ void gemm_tile(const bf16_bits* __restrict__ Ap, int 
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int row = wm * C::WM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-        if (row < a_lim && col < b_lim) Op[(size_t)row * ldo + col] = f32_to_bf16(acc[i][j][v]);
+        if (row < a_lim && col < b_lim) {
+          if constexpr (sizeof(typename C::Elem) == 2) Op[(size_t)row * ldo + col] = f32_to_bf16(acc[i][j][v]);
+          else Op[(size_t)row * ldo + col] = acc[i][j][v];
+        }
       }
     }
   }

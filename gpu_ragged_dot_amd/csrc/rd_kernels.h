@@ -6,6 +6,7 @@
 #include "rd_gemm_w4.h"
 #include "rd_gemm_pp.h"
 #include "rd_gemm_tile.h"
+#include "rd_sched.h"
 
 namespace rd {
 
@@ -18,11 +19,12 @@ struct GmmArgs {
   const int32_t* group_offsets;  // [g]   exclusive prefix sum of group_sizes
   const int32_t* tile2group;     // [U]   scheduling map built with chunk = tile height
   const int32_t* tile2it;        // [U]
+  const int32_t* tile2band;      // [U]   band of row tiles each row tile belongs to (see rd_sched.h)
   const int32_t* total_tiles;    // [1]
   int m, k, n, g;
   int U;        // static bound on row tiles: ceil(m / BM) + g
   int n_tiles;  // ceil(n / BN)
-  int group_m, group_n;  // tiles per L2-sharing block of the tile walk (rows x columns)
+  int group_m, group_n;  // tile walk: most row tiles per band; positions per block = group_m x group_n
   // K-split of the last, partly filled round of tiles (kernels whose configuration has SPLITK; 0 slots = off)
   float* partials;     // [split_slots][BM * BN] fp32
   int32_t* counters;   // [split_slots], zero at launch
@@ -61,26 +63,26 @@ __device__ __forceinline__ void run_tile(const typename C::Elem* Ap, int lda, in
   else if constexpr (C::MIXED) gemm_tile_pingpong_mixed<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
   else if constexpr (C::DLDS && C::PINGPONG) gemm_tile_pingpong<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
   else if constexpr (C::DLDS) gemm_tile_dlds<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
-  else gemm_tile<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
+  else gemm_tile<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, reinterpret_cast<bf16_bits*>(smem));
 }
 
 // How the last round of a gmm launch is cut along K.  The device runs num_cus tiles at a time; when the live tiles do
-// not fill the last round, the row tiles from `first_row` on (the ones that round would hold) are each computed by
-// `parts` work-groups over a `parts`-th of the contraction range instead, so the round takes about 1 / parts as long.
+// not fill the last round, the tiles from position `first_tile` of the walk on (the ones that round would hold) are each
+// computed by `parts` work-groups over a `parts`-th of the contraction range instead, so the round takes about
+// 1 / parts as long.
 struct SplitPlan {
-  int first_row;  // row tiles >= first_row are split; == total when nothing is
+  int first_tile;  // walk positions >= first_tile (and < live) are split; == live when nothing is
   int parts;
-  int tiles;      // (total - first_row) * n_tiles
+  int tiles;       // live - first_tile
 };
 constexpr int kMaxSplitParts = 8;
 constexpr int kMinSplitK = 512;  // contraction elements a piece must keep
 
-__device__ __forceinline__ SplitPlan split_plan(int total, int n_tiles, int k, int slots, int num_cus, int max_parts) {
-  SplitPlan sp{total, 1, 0};
-  if (slots <= 0 || total <= 0) return sp;
-  const int live = total * n_tiles;
-  const int first = ((live / num_cus) * num_cus) / n_tiles;
-  const int tiles = (total - first) * n_tiles;
+__device__ __forceinline__ SplitPlan split_plan(int live, int k, int slots, int num_cus, int max_parts) {
+  SplitPlan sp{live, 1, 0};
+  if (slots <= 0 || live <= 0) return sp;
+  const int first = (live / num_cus) * num_cus;
+  const int tiles = live - first;
   if (tiles <= 0) return sp;
   // The piece that arrives last reads every piece's 256 KB of partial sums at what one compute unit can pull (about
   // 25 GB/s: ~10 us per piece), so the gain of a finer cut, T/parts for a K loop of T us, is soon eaten: parts ~
@@ -96,7 +98,7 @@ __device__ __forceinline__ SplitPlan split_plan(int total, int n_tiles, int k, i
     parts = imin(parts, by_k);
   }
   if (parts < 2) return sp;
-  sp.first_row = first; sp.parts = parts; sp.tiles = tiles;
+  sp.first_tile = first; sp.parts = parts; sp.tiles = tiles;
   return sp;
 }
 
@@ -119,43 +121,53 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
   const E* px = static_cast<const E*>(p.x);
   const E* pA = static_cast<const E*>(p.A);
   E* py = static_cast<E*>(p.y);
-  // Tile walk.  Tiles are grouped into blocks of group_m x group_n (about as many as one XCD runs at a time, so the
-  // block's operand slabs are fetched into that XCD's L2 once), and blocks are dealt to the 8 XCDs (launch index mod 8)
-  // round-robin.  Consecutive row tiles therefore spread over all XCDs, which keeps them evenly loaded when a few
-  // groups are much longer than the rest and their tiles cost more than the mostly-empty ones.
+  // Tile walk.  The scheduling-map kernel has cut every group's row tiles into bands of at most group_m row tiles
+  // (tile2band); the walk visits band after band and, inside a band, column after column (all the band's row tiles of
+  // one column tile, then the next column).  Position t of the walk therefore lies in the band of row tile t / n_tiles.
+  // The walk is cut into blocks of group_m x group_n consecutive positions - a band's rows times a few columns, about
+  // what one XCD runs at a time, so the block's operand slabs are fetched into that XCD's L2 once - and the blocks are
+  // dealt to the 8 XCDs (launch index mod 8) round-robin.  No block spans two groups' weights except where a band ends.
   // Everything read through the map is the same for the whole work-group: pin it to scalar registers.
   const int total = imin(uniform(*p.total_tiles), p.U);
-  SplitPlan sp{total, 1, 0};
-  if constexpr (C::SPLITK) sp = split_plan(total, p.n_tiles, p.k, p.split_slots, p.num_cus, p.max_parts);
+  const int live = total * p.n_tiles;
+  SplitPlan sp{live, 1, 0};
+  if constexpr (C::SPLITK) sp = split_plan(live, p.k, p.split_slots, p.num_cus, p.max_parts);
 
-  int mi, nj;
+  int t;
   SplitK sk;
   int k0 = 0, klen = p.k;
   if ((int)blockIdx.x < p.main_grid) {
     const int per_block = p.group_m * p.group_n;
-    const int block_cols = (p.n_tiles + p.group_n - 1) / p.group_n;
     const int pos = blockIdx.x >> 3;
     const int block = (pos / per_block) * 8 + (blockIdx.x & 7);
-    const int q = pos % per_block;
-    mi = (block / block_cols) * p.group_m + q % p.group_m;
-    nj = (block % block_cols) * p.group_n + q / p.group_m;
-    if (mi >= p.U || nj >= p.n_tiles) return;
-    if (mi >= sp.first_row && mi < total) return;  // computed in pieces by the appended work-groups
+    t = block * per_block + pos % per_block;
+    if (t >= p.U * p.n_tiles) return;
+    if (t >= sp.first_tile && t < live) return;  // computed in pieces by the appended work-groups
   } else {
-    // piece `part` of split tile t; consecutive launch indices take consecutive tiles of one K range
+    // Piece `part` of split tile tt.  The pieces are numbered part-major (all tiles of the first K range, then the
+    // second ...) and every XCD (launch index mod 8) takes one contiguous stretch of that numbering, so that the pieces
+    // an XCD runs together are neighbouring tiles of one K range and share their operand slabs in its L2.
     const int r = blockIdx.x - p.main_grid;
-    if (r >= sp.tiles * sp.parts) return;
-    const int part = r / sp.tiles, t = r - part * sp.tiles;
-    mi = sp.first_row + t / p.n_tiles;
-    nj = t % p.n_tiles;
+    const int pieces = sp.tiles * sp.parts;
+    const int per_xcd = (pieces + 7) >> 3;
+    if ((r >> 3) >= per_xcd) return;
+    const int id = (r & 7) * per_xcd + (r >> 3);
+    if (id >= pieces) return;
+    const int part = id / sp.tiles, tt = id - part * sp.tiles;
+    t = sp.first_tile + tt;
     const int k64 = (p.k + 63) >> 6;
     k0 = (int)((long long)k64 * part / sp.parts) << 6;
     klen = imin(p.k, (int)((long long)k64 * (part + 1) / sp.parts) << 6) - k0;
-    sk.partials = p.partials + (size_t)t * sp.parts * (C::BM * C::BN);
-    sk.counter = p.counters + t;
+    sk.partials = p.partials + (size_t)tt * sp.parts * (C::BM * C::BN);
+    sk.counter = p.counters + tt;
     sk.parts = sp.parts;
     sk.part = part;
   }
+  const int band = uniform(p.tile2band[t / p.n_tiles]);
+  const int band_row0 = band >> kBandShift, band_rows = band & kBandMaxRows;
+  const int w = t - band_row0 * p.n_tiles;
+  const int nj = w / band_rows;
+  const int mi = band_row0 + (w - nj * band_rows);
   const int col0 = nj * C::BN;
   const int cols = imin(C::BN, p.n - col0);
 
@@ -226,7 +238,7 @@ struct TileVariant {
   const char* name;
   int bm, bn, bk, waves_m, waves_n;
   int vec;  // 1: needs k % 8 == 0 and n % 8 == 0 (16-byte row pitches); 0: any shape
-  int f32;     // 1: float32 operands and output; 0: bf16
+  int dtype;   // RD_DTYPE_* of the operands and the output this shape is compiled for
   int dlds;    // 1: direct-to-LDS core (byte extents of one tile's operand window must stay below 2 GiB)
   int stages;  // LDS ring depth
   int splitk;  // 1: the gmm kernels can cut the last round of tiles along K (needs partials in the workspace)
@@ -245,9 +257,10 @@ int launch_gmm(hipStream_t s, const GmmArgs& a) {
   auto kern = gmm_kernel<C, TRANS_RHS>;
   const int attr_rc = allow_big_lds(reinterpret_cast<const void*>(kern), C::LDS_BYTES);
   if (attr_rc != hipSuccess) return attr_rc;
-  const int blocks = ((a.U + a.group_m - 1) / a.group_m) * ((a.n_tiles + a.group_n - 1) / a.group_n);
+  const int per_block = a.group_m * a.group_n;
+  const int blocks = (a.U * a.n_tiles + per_block - 1) / per_block;
   GmmArgs args = a;
-  args.main_grid = 8 * ((blocks + 7) / 8) * a.group_m * a.group_n;
+  args.main_grid = 8 * ((blocks + 7) / 8) * per_block;
   if (!C::SPLITK) args.split_slots = 0;
   const int grid = args.main_grid + args.split_slots;
   if (args.main_grid <= 0) return hipSuccess;

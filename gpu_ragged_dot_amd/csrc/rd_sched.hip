@@ -46,7 +46,8 @@ __global__ __launch_bounds__(kSchedThreads) void sched_map_kernel(const int32_t*
                                                                   int32_t* __restrict__ tile2group,
                                                                   int32_t* __restrict__ tile2it,
                                                                   int32_t* __restrict__ total_tiles,
-                                                                  int32_t* __restrict__ counters, int n_counters) {
+                                                                  int32_t* __restrict__ counters, int n_counters,
+                                                                  int32_t* __restrict__ tile2band, int band_rows) {
   // arrival counters of the K-split tiles of the launch that follows start at zero
   for (int i = threadIdx.x; i < n_counters; i += kSchedThreads) counters[i] = 0;
   __shared__ uint32_t wave_a[kSchedWaves], wave_b[kSchedWaves];
@@ -76,6 +77,17 @@ __global__ __launch_bounds__(kSchedThreads) void sched_map_kernel(const int32_t*
       const int32_t start = l == 0 ? lo : incl[l - 1];
       tile2group[t] = base + l;
       tile2it[t] = t - start;
+      if (tile2band) {
+        // The group's R row tiles are cut into ceil(R / band_rows) bands of nearly equal height (the first R % bands of
+        // them one taller), so that no band spans two groups; the entry says where this tile's band starts and how tall
+        // it is.
+        const int32_t R = incl[l] - start, it = t - start;
+        const int32_t nb = (R + band_rows - 1) / band_rows, r = R / nb, rem = R - r * nb;
+        int32_t row0, rb;
+        if (it < rem * (r + 1)) { rb = r + 1; row0 = (it / rb) * rb; }
+        else { rb = r; row0 = rem * (r + 1) + ((it - rem * (r + 1)) / rb) * rb; }
+        tile2band[t] = ((start + row0) << kBandShift) | rb;
+      }
     }
     carry_rows += ta;
     carry_tiles += tb;
@@ -85,6 +97,7 @@ __global__ __launch_bounds__(kSchedThreads) void sched_map_kernel(const int32_t*
   for (int32_t t = imax((int32_t)carry_tiles, 0) + tid; t < U; t += kSchedThreads) {
     tile2group[t] = 0;
     tile2it[t] = 0;
+    if (tile2band) tile2band[t] = (t << kBandShift) | 1;  // the slots that zero the rows past sum(group_sizes): one-tile bands
   }
   if (tid == 0) *total_tiles = (int32_t)carry_tiles;  // :89
 }
@@ -97,10 +110,13 @@ __global__ void fill_kernel(T* p, size_t n, T v) {
 }  // namespace
 
 int launch_sched_map(hipStream_t s, const int32_t* gs, int g, int m, int chunk, int32_t* group_offsets,
-                     int32_t* tile2group, int32_t* tile2it, int32_t* total_tiles, int32_t* counters, int n_counters) {
+                     int32_t* tile2group, int32_t* tile2it, int32_t* total_tiles, int32_t* counters, int n_counters,
+                     int32_t* tile2band, int band_rows) {
   const int U = (m + chunk - 1) / chunk + g;  // gpu_ragged_dot.py:77
+  if (band_rows < 1) band_rows = 1;
+  if (band_rows > kBandMaxRows) band_rows = kBandMaxRows;
   hipLaunchKernelGGL(sched_map_kernel, dim3(1), dim3(kSchedThreads), 0, s, gs, g, U, chunk, group_offsets,
-                     tile2group, tile2it, total_tiles, counters, counters ? n_counters : 0);
+                     tile2group, tile2it, total_tiles, counters, counters ? n_counters : 0, tile2band, band_rows);
   return (int)hipGetLastError();
 }
 

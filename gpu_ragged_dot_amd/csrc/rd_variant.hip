@@ -1,5 +1,6 @@
 // One compiled tile shape.  Built once per entry of the variant list in the Makefile, with
-//   -DRD_BM= -DRD_BN= -DRD_BK= -DRD_WAVES_M= -DRD_WAVES_N= -DRD_VEC= -DRD_NAME= [-DRD_DLDS=1|2 -DRD_STAGES= -DRD_PINGPONG=1]
+//   -DRD_BM= -DRD_BN= -DRD_BK= -DRD_WAVES_M= -DRD_WAVES_N= -DRD_VEC= -DRD_NAME= [-DRD_DLDS=1|2|3 -DRD_STAGES= -DRD_PINGPONG=1
+//   -DRD_F32=1|2]
 // and exports a getter rd_variant_<name>() for its TileVariant record that the C-ABI file collects.
 #include "rd_kernels.h"
 
@@ -23,7 +24,12 @@
 #endif
 
 namespace rd {
-#if RD_F32
+#if RD_F32 == 2
+// float32 arrays, rounded to bf16 on the way into LDS, bf16 matrix cores, float32 out (compute_dtype = bfloat16)
+typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, /*A K-major*/ true, /*B K-major*/ false, RD_VEC != 0, float> CfgNN;
+typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, true, true, RD_VEC != 0, float> CfgNT;
+typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, false, false, RD_VEC != 0, float> CfgTN;
+#elif RD_F32
 typedef F32Cfg<RD_BM, RD_BN, /*A K-major*/ true, /*B K-major*/ false> CfgNN;
 typedef F32Cfg<RD_BM, RD_BN, true, true> CfgNT;
 typedef F32Cfg<RD_BM, RD_BN, false, false> CfgTN;
@@ -51,7 +57,7 @@ typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, false, false, RD_VE
 
 extern "C" const rd::TileVariant* RD_CAT(rd_variant_, RD_NAME)() {
   static const rd::TileVariant v = {
-      RD_STR(RD_NAME), RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, RD_VEC, RD_F32, RD_DLDS != 0, RD_STAGES,
+      RD_STR(RD_NAME), RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, RD_VEC, /*dtype: RD_DTYPE_* */ RD_F32, RD_DLDS != 0, RD_STAGES,
       /*splitk*/ RD_DLDS != 0 && !RD_F32,
       &rd::launch_gmm<rd::CfgNN, false>, &rd::launch_gmm<rd::CfgNT, true>, &rd::launch_tgmm<rd::CfgTN>};
   return &v;

@@ -21,13 +21,26 @@ _DTYPES = {torch.bfloat16: _capi.RD_DTYPE_BF16, torch.float32: _capi.RD_DTYPE_F3
 
 
 def _dtype_code(t: torch.Tensor, compute_dtype, acc_dtype) -> int:
+    """Element-type code for the C ABI from the storage dtype and the reference's ``compute_dtype``
+    (gpu_ragged_dot.py:116-119, 145: operands are cast to compute_dtype before the dot; None = the storage dtype)."""
     if t.dtype not in _DTYPES:
         raise TypeError(f"unsupported dtype {t.dtype}; operands are bfloat16 or float32")
-    if compute_dtype is not None and compute_dtype != t.dtype:
-        raise NotImplementedError(f"compute_dtype={compute_dtype} differs from the operand dtype {t.dtype}")
     if acc_dtype not in (None, torch.float32):
         raise NotImplementedError("accumulation is always float32 on the matrix cores")
-    return _DTYPES[t.dtype]
+    if compute_dtype is None or compute_dtype == t.dtype:
+        return _DTYPES[t.dtype]
+    if t.dtype == torch.float32 and compute_dtype == torch.bfloat16:
+        return _capi.RD_DTYPE_F32_BF16  # rounded to bf16 on the way to the bf16 matrix cores, float32 out
+    if t.dtype == torch.bfloat16 and compute_dtype == torch.float32:
+        # widening bf16 operands changes nothing: their products are exact in fp32 and accumulation is fp32 anyway
+        return _capi.RD_DTYPE_BF16
+    raise NotImplementedError(f"no kernel for compute_dtype={compute_dtype} on {t.dtype} operands")
+
+
+def _aligned16(*tensors: torch.Tensor) -> bool:
+    """The fast tile shapes move 16 bytes at a time: every buffer must start on a 16-byte boundary (a view at an odd
+    element offset does not, however contiguous it is)."""
+    return all(t.data_ptr() % 16 == 0 for t in tensors)
 
 
 def _check_device(*tensors: torch.Tensor) -> torch.device:
@@ -82,7 +95,7 @@ def _gmm_fwd(x, A, group_sizes, block_m, block_k, block_n, trans_rhs, interpret,
     y = torch.empty((m, n), dtype=x.dtype, device=dev)  # :210
     if plan is None:
         plan = planner.select_plan(_capi.OP_GMM_TRANS if trans_rhs else _capi.OP_GMM, m, k, n, g, block_m, block_k, block_n,
-                                   dtype=code)
+                                   dtype=code, aligned=_aligned16(x, A, y))
     ws_bytes = _capi.lib.rd_gmm_workspace_bytes(m, g, _plan_ref(plan))
     ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
@@ -112,7 +125,8 @@ def _tgmm_fwd(x, y, group_sizes, block_m, block_k, block_n, interpret, compute_d
     gs = _group_sizes_i32(gs_t, dev)
     out = torch.empty((g, k, n), dtype=x.dtype, device=dev)  # :324
     if plan is None:
-        plan = planner.select_plan(_capi.OP_TGMM, m, k, n, g, block_m, block_k, block_n, dtype=code)
+        plan = planner.select_plan(_capi.OP_TGMM, m, k, n, g, block_m, block_k, block_n, dtype=code,
+                                   aligned=_aligned16(x, y, out))
     ws_bytes = _capi.lib.rd_tgmm_workspace_bytes(m, g, _plan_ref(plan))
     ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):

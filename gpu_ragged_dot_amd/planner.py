@@ -90,10 +90,19 @@ def select_plan(
     block_k: int = DEFAULT_BLOCK_K,
     block_n: int = DEFAULT_BLOCK_N,
     dtype: int = _capi.RD_DTYPE_BF16,
+    aligned: bool = True,
 ) -> _capi.Plan:
-    """Plan for op (0 gmm, 1 gmm with trans_rhs, 2 tgmm) on a problem of this shape and element type."""
+    """Plan for op (0 gmm, 1 gmm with trans_rhs, 2 tgmm) on a problem of this shape and element type.
+
+    ``aligned``: every buffer of the call starts on a 16-byte boundary.  When one does not, the plan is the
+    element-granular tile shape of that element type, whatever the shape, the tuned table or block_* ask for."""
+    if not aligned and dtype != _capi.RD_DTYPE_F32:
+        for v in compiled_variants():
+            if v.dtype == dtype and not v.vec:
+                return _capi.Plan(v.id)
+        raise _capi.RaggedDotError(_capi.RD_ERR_UNSUPPORTED, "no any-alignment tile shape compiled in for this dtype")
     if dtype != _capi.RD_DTYPE_BF16:
-        return _capi.default_plan(op, m, k, n, g, dtype)  # one float32 kernel: nothing to choose
+        return _capi.default_plan(op, m, k, n, g, dtype)  # the library's own choice: nothing to tune
     vec = k % 8 == 0 and n % 8 == 0
     explicit = (block_m, block_k, block_n) != (DEFAULT_BLOCK_M, DEFAULT_BLOCK_K, DEFAULT_BLOCK_N)
     entry = tuned_plans().get(plan_key(op, m, k, n, g))

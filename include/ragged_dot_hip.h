@@ -27,7 +27,12 @@ extern "C" {
 
 #define RD_ABI_VERSION 2
 
-enum rd_dtype { RD_DTYPE_BF16 = 0, RD_DTYPE_F32 = 1 };
+/* Element type of the operands and the output (always the same, gpu_ragged_dot.py:210,324) and what the matrix cores
+ * multiply.  RD_DTYPE_F32_BF16 is compute_dtype = bfloat16 on float32 arrays (gpu_ragged_dot.py:116-119, 145, 149): the
+ * float32 elements are rounded to bfloat16 (nearest even) as they are loaded, multiplied on the bf16 matrix cores with
+ * fp32 accumulation, and stored as float32.  (compute_dtype = float32 on bfloat16 arrays is RD_DTYPE_BF16 itself: a
+ * product of two bfloat16 values is exact in fp32, and the accumulation is fp32 either way.) */
+enum rd_dtype { RD_DTYPE_BF16 = 0, RD_DTYPE_F32 = 1, RD_DTYPE_F32_BF16 = 2 };
 
 #define RD_DECODE_ROWS (-1) /* rd_plan.decode_nb: the streaming kernel that cuts each expert's weights into whole-row slices */
 
@@ -54,8 +59,10 @@ typedef struct rd_variant_info {
 /* Launch plan for one call; the host planner (or the caller) fills it.  variant = -1 with every other field 0 = library defaults. */
 typedef struct rd_plan {
   int variant; /* index into the variant table, or -1: let the library choose by shape */
-  int group_m; /* tile walk: row tiles per L2-sharing block (tgmm: per band); 0 = default */
-  int group_n; /* tile walk: column tiles per block (rd_gmm only); 0 = default */
+  int group_m; /* tile walk.  rd_gmm: a group's row tiles are cut into bands of at most group_m (1..127) row tiles and the
+                  walk goes band by band, column by column inside a band.  rd_tgmm: row tiles per band.  0 = default */
+  int group_n; /* rd_gmm only: the walk is dealt to the 8 XCDs in blocks of group_m x group_n (<= 4096) consecutive tiles;
+                  the product should equal what one XCD runs at a time (32 for the 256 x 256 tiles).  0 = default */
   int decode_nb; /* rd_gmm only, for a few rows per group: > 0 selects the streaming kernel that gives each work-group
                     this many columns (32, 64 or 128) of one expert; RD_DECODE_ROWS the one that gives it whole rows
                     for a slice of the contraction range (fp32 partial sums in the workspace, n <= 2048) */

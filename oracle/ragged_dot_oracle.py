@@ -22,6 +22,8 @@ Every function names the reference lines it restates.  How each one is pinned
 * ``gmm_vjp`` - adjoint identities <dout, gmm(x,A)> = <dlhs, x> = <drhs, A> in
   float64, which fix the wiring of gpu_ragged_dot.py:400-401 with no outside
   oracle, plus central finite differences.
+* ``tgmm_vjp`` - the same two checks for s(x, y) = <dout, tgmm(x, y)>:
+  <dx, x> = <dy, y> = s, and central differences along random directions.
 * block-size rules - table tests of the integer rules.
 
 The reference holds no golden vectors or fixtures on disk (tests.py compares
@@ -191,6 +193,17 @@ def gmm_vjp(x, A, group_sizes, dout, trans_rhs: bool = False, out_dtype: str = "
     else:
         dA = tgmm(dout, x, group_sizes, out_dtype=out_dtype, acc=acc)
     return dx, dA, None
+
+
+def tgmm_vjp(x, y, group_sizes, dout, out_dtype: str = "bfloat16", acc=np.float32):
+    """VJP of tgmm(x, y) = per-group x_g^T y_g with cotangent dout[g, k, n]: what gpu_ragged_dot.py:431-450 means to
+    compute.  dx = gmm(y, dout, trans_rhs=True) (rows of group g: y_g @ dout[g].T, as :444-446), and
+    dy = gmm(x, dout) (rows of group g: x_g @ dout[g]).  The reference writes the latter as tgmm(x, do) (:447-449),
+    which cannot run (a 3-D `do` fails the y.ndim == 2 assert of :304); the product restated here is the one the
+    mathematics fixes - pinned by adjoint identities and central differences, not by the reference's text."""
+    dx = gmm(y, dout, group_sizes, trans_rhs=True, out_dtype=out_dtype, acc=acc)
+    dy = gmm(x, dout, group_sizes, trans_rhs=False, out_dtype=out_dtype, acc=acc)
+    return dx, dy, None
 
 
 # ---------------------------------------------------------------------------------------------------------------------

@@ -205,6 +205,33 @@ def test_vjp_adjoint_identities_and_finite_differences(trans_rhs):
     assert not np.any(dx[27:]) and not np.any(dA[1])
 
 
+def test_tgmm_vjp_adjoint_identities_and_finite_differences():
+    """The VJP of tgmm (what gpu_ragged_dot.py:431-450 intends): s(x, y) = <dout, tgmm(x, y)> is bilinear, so
+    <dx, x> = <dy, y> = s, and its directional derivatives are <dx, vx> and <dy, vy>.  A swapped operand, a missing
+    transpose or cotangents leaking into rows past sum(group_sizes) fails one of these."""
+    rng = np.random.default_rng(6)
+    m, k, n, g = 30, 7, 5, 4
+    gs = [8, 0, 15, 4]  # 27 of 30 rows used, one empty group
+    x, y = rng.normal(size=(m, k)), rng.normal(size=(m, n))
+    dout = rng.normal(size=(g, k, n))
+    f = lambda x_, y_: oracle.tgmm(x_, y_, gs, out_dtype="float32", acc=np.float64)
+    dx, dy, dgs = oracle.tgmm_vjp(x, y, gs, dout, out_dtype="float32", acc=np.float64)
+    assert dgs is None and dx.shape == x.shape and dy.shape == y.shape
+    s = np.sum(dout * f(x, y))
+    np.testing.assert_allclose(np.sum(dx * x), s, rtol=1e-10)
+    np.testing.assert_allclose(np.sum(dy * y), s, rtol=1e-10)
+    vx, vy = rng.normal(size=x.shape), rng.normal(size=y.shape)
+    eps = 1e-6
+    num_x = (np.sum(dout * f(x + eps * vx, y)) - np.sum(dout * f(x - eps * vx, y))) / (2 * eps)
+    num_y = (np.sum(dout * f(x, y + eps * vy)) - np.sum(dout * f(x, y - eps * vy))) / (2 * eps)
+    np.testing.assert_allclose(np.sum(dx * vx), num_x, rtol=1e-6)
+    np.testing.assert_allclose(np.sum(dy * vy), num_y, rtol=1e-6)
+    assert not np.any(dx[27:]) and not np.any(dy[27:])
+    # per group, by the definition: dx_g = y_g dout_g^T, dy_g = x_g dout_g
+    np.testing.assert_allclose(dx[8:23], y[8:23] @ dout[2].T, rtol=1e-12)
+    np.testing.assert_allclose(dy[23:27], x[23:27] @ dout[3], rtol=1e-12)
+
+
 # ---- the loop-nest restatement against the definition, on the reference's own grid ----------------------------------
 
 GRID = util.reference_grid(36, seed=1)
