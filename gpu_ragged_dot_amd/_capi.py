@@ -78,6 +78,8 @@ EXPORTS = (
     "rd_sched_map_len",
     "rd_gmm_workspace_bytes",
     "rd_gmm",
+    "rd_gmm_noalloc_scratch_bytes",
+    "rd_gmm_noalloc",
     "rd_tgmm_workspace_bytes",
     "rd_tgmm",
     "rd_moe_route_workspace_bytes",
@@ -116,6 +118,10 @@ def _load() -> ctypes.CDLL:
     lib.rd_gmm_workspace_bytes.restype = sz
     lib.rd_gmm.argtypes = [vp, vp, vp, ip, vp, i, i, i, i, i, i, ctypes.POINTER(Plan), vp, sz]
     lib.rd_gmm.restype = i
+    lib.rd_gmm_noalloc_scratch_bytes.argtypes = []
+    lib.rd_gmm_noalloc_scratch_bytes.restype = sz
+    lib.rd_gmm_noalloc.argtypes = [vp, vp, vp, ip, vp, i, i, i, i, i, i, ctypes.POINTER(Plan)]
+    lib.rd_gmm_noalloc.restype = i
     lib.rd_tgmm_workspace_bytes.argtypes = [i, i, ctypes.POINTER(Plan)]
     lib.rd_tgmm_workspace_bytes.restype = sz
     lib.rd_tgmm.argtypes = [vp, vp, vp, ip, vp, i, i, i, i, i, ctypes.POINTER(Plan), vp, sz]

@@ -105,6 +105,19 @@ int rd_gmm(void* stream, const void* x, const void* A, const int32_t* group_size
            int g, int trans_rhs, int dtype, const rd_plan* plan /* host, may be NULL */, void* workspace,
            size_t workspace_bytes);
 
+/* ---- rd_gmm without a workspace -------------------------------------------------------------------------------
+ * No counterpart in the reference.  For callers that cannot allocate device memory: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  Same product as rd_gmm, same kernels; what rd_gmm keeps in the
+ * caller's workspace (the scheduling map, the streaming kernel's partial sums) lives in a buffer of
+ * rd_gmm_noalloc_scratch_bytes() = 4 MiB built into the library, one copy per device, held until the process ends.
+ * The call allocates and frees nothing.  Limits: the scheduling map must fit (rd_gmm_workspace_bytes(m, g, plan with
+ * split_k = -1) <= 4 MiB, i.e. roughly m / 16 + g <= 349 000), otherwise RD_ERR_WORKSPACE; the K-split is never used.
+ * All calls on one device share that device's buffer: calls that overlap on one device (different streams, or
+ * different threads without stream ordering between them) race; calls ordered on one stream do not. */
+size_t rd_gmm_noalloc_scratch_bytes(void);
+int rd_gmm_noalloc(void* stream, const void* x, const void* A, const int32_t* group_sizes, void* y, int m, int k, int n,
+                   int g, int trans_rhs, int dtype, const rd_plan* plan /* host, may be NULL */);
+
 /* ---- tgmm: dA[g, k, n] = x[rows of g, :]^T . dy[rows of g, :] -----------------------------------------------
  * Replaces the "gpu_tgmm" pallas_call (gpu_ragged_dot.py:231-281, 331-340).  Slices of empty groups are zero
  * (:277-281).  x is [m, k], dy is [m, n]. */
