@@ -9,7 +9,10 @@ from __future__ import annotations
 import ctypes
 import os
 
-import torch  # noqa: F401  - loaded first so the HIP runtime already in the process is the one the library binds to
+try:  # loaded first, when present, so that the HIP runtime already in the process is the one the library binds to
+    import torch  # noqa: F401
+except ImportError:  # a JAX-only process: the library then loads the system HIP runtime, as jaxlib's ROCm plugin does
+    torch = None
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libragged_dot_hip.so")
