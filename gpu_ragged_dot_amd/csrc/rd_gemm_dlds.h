@@ -15,14 +15,16 @@
 
 namespace rd {
 
+// B_AUX: cache policy of the B operand's loads (0 = default, kCachePolicyStream = read once, do not keep in L2).
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, bool A_KMAJOR_, bool B_KMAJOR_, int STAGES_,
-          bool PINGPONG_ = false>
+          bool PINGPONG_ = false, int B_AUX_ = 0>
 struct DldsCfg {
   typedef bf16_bits Elem;
   static constexpr bool F32 = false;
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
   static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = true, DLDS = true, PINGPONG = PINGPONG_, MIXED = false,
                         SPLITK = true;
+  static constexpr int B_AUX = B_AUX_;
   static constexpr int NW = WAVES_M * WAVES_N;
   static constexpr int NT = 64 * NW;
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
@@ -41,7 +43,8 @@ struct DldsCfg {
   static constexpr int RING_BYTES = STAGES * STAGE_BYTES;
   static constexpr int LDS_BYTES = RING_BYTES > EPI_BYTES ? RING_BYTES : EPI_BYTES;
   static_assert(BK == 64 || BK == 32, "contraction slab");
-  static_assert(BM % 128 == 0 && BN % 128 == 0, "direct-to-LDS tiles are at least 128 wide");
+  // an MN-major slab row holds the operand's whole tile extent and its chunk permutation needs 16 chunks (128 elements)
+  static_assert((A_KMAJOR ? BM % 64 == 0 : BM % 128 == 0) && BN % 128 == 0, "direct-to-LDS tile extents");
   static_assert(BM % (32 * WAVES_M) == 0 && BN % (32 * WAVES_N) == 0, "tile shape");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
   static_assert(!PINGPONG || (NW == 8 && WAVES_M == 2 && STAGES >= 3), "ping-pong runs two groups of four waves");
@@ -51,6 +54,7 @@ typedef __attribute__((address_space(3))) void* lds_void_ptr;
 
 constexpr int kBufferFlags = 0x00020000;   // raw buffer, 32-bit data format
 constexpr int kOobOffset = 0x7ffffff0;     // byte offset past any buffer: the load returns zeros
+constexpr int kCachePolicyStream = 2;      // nt in the aux operand of the buffer intrinsics: streamed data, first to be evicted
 
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -59,7 +63,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 }
 
 // One operand's slab loader: which 16 bytes each lane fetches for each of its wave's load instructions.
-template <int T, int BK, int NW, bool KMAJOR>
+template <int T, int BK, int NW, bool KMAJOR, int AUX = 0>
 struct DldsLoader {
   static constexpr int ROW_BYTES = KMAJOR ? BK * 2 : T * 2;
   static constexpr int RPI = 1024 / ROW_BYTES;   // slab rows per wave-wide load
@@ -113,7 +117,7 @@ struct DldsLoader {
                                         int klen) const {
     int off = voff[j];
     if (TAIL && KMAJOR && k0 + kcol >= klen) off = kOobOffset;  // MN-major tails are out of `records` by themselves
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(lds + (wave + NW * j) * 1024), 16, off, 0, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(lds + (wave + NW * j) * 1024), 16, off, 0, 0, AUX);
   }
 
   __device__ __forceinline__ void advance() {
@@ -283,7 +287,7 @@ __device__ __forceinline__ void gemm_tile_dlds(const bf16_bits* __restrict__ Ap,
   const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;
 
   typedef DldsLoader<C::BM, C::BK, C::NW, C::A_KMAJOR> LdA;
-  typedef DldsLoader<C::BN, C::BK, C::NW, C::B_KMAJOR> LdB;
+  typedef DldsLoader<C::BN, C::BK, C::NW, C::B_KMAJOR, C::B_AUX> LdB;
   LdA la; LdB lb;
   la.init(Ap, lda, a_lim, klen, wave, lane);
   lb.init(Bp, ldb, b_lim, klen, wave, lane);

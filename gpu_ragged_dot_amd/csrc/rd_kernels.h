@@ -66,6 +66,23 @@ __device__ __forceinline__ void run_tile(const typename C::Elem* Ap, int lda, in
   else gemm_tile<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, reinterpret_cast<bf16_bits*>(smem));
 }
 
+// Row tiles of a group with at most kShortRows rows (most tiles of a launch when the groups are much shorter than the
+// tile: a mixture of experts with a few dozen tokens per expert).  Such a tile is a stream over its 256 columns of the
+// group's weights with next to no matrix-core work, so what counts is how many bytes each compute unit keeps in flight
+// and that every load covers whole 128-byte lines: the same 256 threads run a 64-row tile routine instead, whose LDS
+// ring holds only 4-8 KB of activations per slab - 8 slabs of 32 deep for weights read across rows (7 x 20 KB requested
+// ahead of use against 3.5 x 32 KB in the tall routine), 4 slabs of 64 deep for weights read along rows.  The weights
+// of such a group are read by this one row tile only: they are streamed past L2 (nt), which keeps L2 for what the
+// tall tiles of long groups share.
+// A 128-row routine of the same kind (6 slabs of 32, or 3 of 64) serves the tiles with 65 to 128 rows.
+constexpr int kShortRows = 64, kMidRows = 128;
+template <class C, int ROWS>
+struct ShortTileCfg {
+  static constexpr int BK = C::B_KMAJOR ? 64 : 32;
+  static constexpr int STAGES = (160 * 1024) / ((ROWS + C::BN) * BK * 2);
+  typedef DldsCfg<ROWS, C::BN, BK, 1, 4, true, C::B_KMAJOR, STAGES, false, kCachePolicyStream> type;
+};
+
 // How the last round of a gmm launch is cut along K.  The device runs num_cus tiles at a time; when the live tiles do
 // not fill the last round, the tiles from position `first_tile` of the walk on (the ones that round would hold) are each
 // computed by `parts` work-groups over a `parts`-th of the contraction range instead, so the round takes about
@@ -182,6 +199,18 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
     const E* Bp = TRANS_RHS ? pA + (size_t)gi * p.n * p.k + (size_t)col0 * p.k + k0
                             : pA + (size_t)gi * p.k * p.n + (size_t)k0 * p.n + col0;
     E* Op = py + (size_t)row0 * p.n + col0;
+    if constexpr (IsW4<C>::value && C::A_KMAJOR) {
+      // only a group's single row tile: the weights of a longer group are shared by its row tiles through L2
+      if (rows <= kMidRows && it == 0) {
+        typedef typename ShortTileCfg<C, kShortRows>::type S;
+        typedef typename ShortTileCfg<C, kMidRows>::type M;
+        static_assert(S::LDS_BYTES <= C::LDS_BYTES && S::NT == C::NT && S::BN == C::BN, "the short routine runs in the tall one's launch");
+        static_assert(M::LDS_BYTES <= C::LDS_BYTES && M::NT == C::NT && M::BN == C::BN, "the 128-row routine runs in the tall one's launch");
+        if (rows <= kShortRows) gemm_tile_dlds<S>(Ap, p.k, rows, Bp, TRANS_RHS ? p.k : p.n, cols, klen, Op, p.n, smem, sk);
+        else gemm_tile_dlds<M>(Ap, p.k, rows, Bp, TRANS_RHS ? p.k : p.n, cols, klen, Op, p.n, smem, sk);
+        return;
+      }
+    }
     run_tile<C>(Ap, p.k, rows, Bp, TRANS_RHS ? p.k : p.n, cols, klen, Op, p.n, smem, sk);
   } else {
     // Rows past sum(group_sizes) are defined to be zero.  The map never uses more than

@@ -332,3 +332,40 @@ def test_k_split_workspace_reused_across_shapes():
         util.assert_close_rows(outs[0], oracle.gmm(lhs, rhs, gs), target_m, util.BF16_EPS, "split y")
         scale = np.abs(outs[1]).max()
         assert np.abs(outs[0] - outs[1]).max() <= 2 ** -7 * scale
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# the streaming routines for row tiles of short groups inside the 256 x 256 four-wave kernel
+# ---------------------------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("trans_rhs", [False, True], ids=["A", "At"])
+@pytest.mark.parametrize("k,split_k", [(72, -1), (1096, -1), (4104, 8), (2048, 3)], ids=["k72", "k1096", "k4104-split8", "k2048-split3"])
+def test_short_group_row_tiles(k, split_k, trans_rhs):
+    """Groups of 1..64 rows (64-row streaming routine), 65..128 rows (128-row routine), 129..256 and longer (tall
+    routine, also for the short last tile of a long group) in one launch of the four-wave kernel, with contraction
+    lengths that end inside a slab, and with the K-split cutting those tiles too."""
+    vid = [v.id for v in _capi.variants() if v.name.decode().startswith("w256")][0]
+    gs = np.array([5, 64, 65, 128, 129, 0, 33, 100, 1, 256, 300, 257, 640], np.int32)
+    m, n, g = int(gs.sum()) + 40, 520, gs.size
+    print(f"short tiles k={k} split_k={split_k} trans_rhs={trans_rhs}", flush=True)
+    lhs, rhs, _, _, _ = util.make_case(k, m, k, n, g, 1.0, True, scale_rhs=True)
+    target_m = int(gs.sum())
+    x = util.bf16_dev(lhs)
+    A = util.bf16_dev(np.ascontiguousarray(np.swapaxes(rhs, 1, 2)) if trans_rhs else rhs)
+    gs_d = torch.from_numpy(gs).cuda()
+    plan = _capi.Plan(vid, 2, 0, 4, split_k=split_k)
+    ws = torch.empty(_capi.lib.rd_gmm_workspace_bytes(m, g, ctypes.byref(plan)), dtype=torch.uint8, device="cuda")
+    ws.fill_(0x3C)
+    y_ref = oracle.gmm(lhs, rhs, gs)
+    prev = None
+    for _ in range(2):
+        y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        rc = _capi.lib.rd_gmm(_stream(), x.data_ptr(), A.data_ptr(), gs_d.data_ptr(), y.data_ptr(), m, k, n, g,
+                              int(trans_rhs), _capi.RD_DTYPE_BF16, ctypes.byref(plan), ws.data_ptr(), ws.numel())
+        assert rc == 0, _capi.lib.rd_last_error()
+        torch.cuda.synchronize()
+        assert not torch.isnan(y).any()
+        util.assert_close_rows(util.to_np(y), y_ref, target_m, util.BF16_EPS, "y")
+        assert not torch.any(y[target_m:])
+        assert prev is None or torch.equal(prev, y)
+        prev = y
