@@ -1,15 +1,21 @@
 """Throughput of the ragged_dot hot path on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--only] [--no-cpu-baseline]
 
 One step = one pass of the hot path over one synthetic batch already resident in HBM: forward for the forward-only
-workloads, forward + dlhs + drhs for the others.  Prints one JSON line (see the keys below).  The default workload is
-the Mixtral-8x7B-shaped forward+backward.
+workloads, forward + dlhs + drhs for the others.  Prints ONE JSON line.  Its top-level keys describe the headline
+workload (default: the Mixtral-8x7B-shaped forward+backward).  Unless --only is given, the same line also carries
+  "configs": the other measured configurations (mixtral_fwd, deepseek_fwd_bwd, decode), each with ms_per_step, value,
+             roofline and cpu_baseline of its own;
+  "context": what the same box does with a dense bf16 GEMM of the Mixtral forward's size (torch.matmul, on N(0,1)
+             data and on zeros), a sustained (>= 2 s) loop of the headline step, a bare read of the decode shape's
+             bytes, and the CPU model.
 """
 
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -19,10 +25,14 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2516.6  # dense bf16 MFMA: 256 CU x 4 SIMD x 1024 FLOP/clk x 2.4 GHz
 PEAK_HBM_GBS = 8000.0
+DEFAULT_WORKLOAD = "mixtral_fwd_bwd"
+OTHER_CONFIGS = ("mixtral_fwd", "deepseek_fwd_bwd", "decode")
+HP = dict(block_m=64, block_k=64, block_n=64, interpret=False, compute_dtype=None, chunk_m=512)
 
 
 def _event_ms(fn, reps, torch):
-    """Average milliseconds per call of fn() over `reps` back-to-back calls, by events on the launch stream."""
+    """Average milliseconds per call of fn() over `reps` back-to-back calls, by events on the launch stream (every
+    kernel of the library is enqueued on torch's current stream, which is the one the events are recorded on)."""
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for _ in range(reps):
@@ -32,7 +42,18 @@ def _event_ms(fn, reps, torch):
     return start.elapsed_time(stop) / reps
 
 
-def cpu_baseline(name, seconds_hint=20.0):
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(name, seconds_hint):
     """The numpy oracle on this host's cores, on a bounded sample of the same workload: whole groups (all their rows,
     the full k and n), forward (+ backward where the workload has one), until about `seconds_hint` of work is done."""
     import numpy as np
@@ -70,18 +91,204 @@ def cpu_baseline(name, seconds_hint=20.0):
         "value": value,
         "unit": unit,
         "cores": cores,
+        "cpu": cpu_model(),
         "kind": "port",
         "sample": f"numpy oracle (fp32 BLAS per group) on {len(used)} whole group(s) of '{name}' "
                   f"({sum(int(gs[i]) for i in used)} rows), {elapsed:.1f} s",
     }
 
 
+def _plan_text(plan, planner):
+    if plan.decode_nb:
+        return "decode_rows" if plan.decode_nb < 0 else "decode_nb%d" % plan.decode_nb
+    return "%s:%d:%d" % (planner.compiled_variants()[plan.variant].name.decode(), plan.group_m, plan.group_n)
+
+
+def measure(name, steps, warmup, torch, sustained_seconds=0.0, headline=False):
+    """One workload: inputs on the device, `warmup` untimed steps, then exactly `steps` timed steps between events;
+    per-product launch durations and the roofline of the dominant one."""
+    import gpu_ragged_dot_amd  # noqa: F401
+    from gpu_ragged_dot_amd import ops, planner, workloads
+
+    w = workloads.WORKLOADS[name]
+    dev = torch.device("cuda:0")
+    x, A, dout, gs = workloads.make_inputs(name, device=dev)
+    hp = dict(HP, acc_dtype=torch.float32)
+    if name == "decode" and not headline:  # a 35 us step: more of them (the headline keeps exactly the steps it was given)
+        steps, warmup = max(steps * 10, 200), max(warmup, 20)
+
+    # For the memory-bound decode shape the 167 MB of expert weights would otherwise sit in the 256 MB last-level
+    # cache between steps: rotate over several copies so that every step streams from HBM.
+    copies = [A] + ([A.clone() for _ in range(5)] if name == "decode" else [])
+    state = {"i": 0}
+
+    def fwd():
+        a = copies[state["i"] % len(copies)]
+        state["i"] += 1
+        return ops._gmm_fwd(x, a, gs, **hp, trans_rhs=False)
+
+    def dlhs():
+        return ops._gmm_fwd(dout, A, gs, **hp, trans_rhs=True)
+
+    def drhs():
+        return ops._tgmm_fwd(x, dout, gs, **hp)
+
+    parts = [("fwd", fwd)] + ([("dlhs", dlhs), ("drhs", drhs)] if w.backward else [])
+
+    def step():
+        for _, fn in parts:
+            fn()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ms_per_step = _event_ms(step, steps, torch)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    # The decode step is one ~35 us call: also time it replayed from a HIP graph (one graph = one call per weight
+    # copy), which takes the host's launch path out of the measurement.
+    graph_ms = None
+    if name == "decode":
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for a in copies:
+                ops._gmm_fwd(x, a, gs, **hp, trans_rhs=False)
+        for _ in range(3):
+            graph.replay()
+        graph_ms = _event_ms(graph.replay, max(steps // len(copies), 4), torch) / len(copies)
+
+    # per-product launch durations, for the roofline of the dominant kernel
+    if len(parts) == 1:  # the step is that one product: the timed region already is its launch duration
+        per = {parts[0][0]: ms_per_step}
+    else:
+        per = {pname: _event_ms(fn, max(steps, 5), torch) for pname, fn in parts}
+    dominant = max(per, key=per.get)
+    flops_step = workloads.flops(name)
+    abytes = workloads.algorithmic_bytes(name)
+    flops_one = flops_step / (3 if w.backward else 1)
+
+    if name == "decode":
+        metric, unit = "ragged_dot decode forward, expert weights streamed", "GB/s"
+        value = abytes["weights_read"] / (ms_per_step * 1e-3) / 1e9
+        roof = {"bound": "hbm", "achieved": abytes[dominant] / (per[dominant] * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                "unit": "GB/s"}
+    else:
+        metric, unit = ("ragged_dot fwd+bwd" if w.backward else "ragged_dot fwd") + " throughput", "TFLOP/s"
+        value = flops_step / (ms_per_step * 1e-3) / 1e12
+        t_flop = flops_one / (PEAK_BF16_TFLOPS * 1e12)
+        t_byte = abytes[dominant] / (PEAK_HBM_GBS * 1e9)
+        if t_byte > t_flop:
+            roof = {"bound": "hbm", "achieved": abytes[dominant] / (per[dominant] * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                    "unit": "GB/s"}
+        else:
+            roof = {"bound": "mfma", "achieved": flops_one / (per[dominant] * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
+                    "unit": "TFLOP/s"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+
+    plans = {}
+    for pname, op, (mm, kk, nn) in (("fwd", 0, (w.m, w.k, w.n)), ("dlhs", 1, (w.m, w.n, w.k)), ("drhs", 2, (w.m, w.k, w.n))):
+        if pname in per:
+            plans[pname] = _plan_text(planner.select_plan(op, mm, kk, nn, w.g), planner)
+
+    # HBM bytes per launch of the dominant kernel, from the committed counter runs (profiles/hbm_traffic.json).  Each
+    # figure there is tagged with the plan it was measured under; a figure for another plan is stale and not reported.
+    roof["traffic"] = None
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            entry = json.load(f).get(name, {}).get(dominant)
+        if isinstance(entry, dict) and entry.get("plan") == plans.get(dominant):
+            roof["traffic"] = entry.get("bytes")
+    except (OSError, ValueError):
+        pass
+    roof["kernel"] = {"fwd": "gmm_kernel<.., trans_rhs=false>" if name != "decode" else "gmm_rows_kernel + gmm_rows_finish_kernel",
+                      "dlhs": "gmm_kernel<.., trans_rhs=true>", "drhs": "tgmm_kernel"}[dominant]
+    roof["launch_ms"] = per[dominant]
+    roof["algorithmic_per_launch"] = abytes[dominant] if roof["bound"] == "hbm" else flops_one
+
+    out = {
+        "metric": metric,
+        "value": value,
+        "unit": unit,
+        "ms_per_step": ms_per_step,
+        "steps": steps,
+        "warmup": warmup,
+        "config": {"workload": name, "m": w.m, "k": w.k, "n": w.n, "g": w.g, "backward": w.backward,
+                   "description": w.description, "group_sizes": "seeded, see gpu_ragged_dot_amd/workloads.py"},
+        "frac_of_bf16_mfma_peak": (value / PEAK_BF16_TFLOPS) if unit == "TFLOP/s" else None,
+        "frac_of_step_roofline": None,
+        "per_kernel_ms": per,
+        "graph_replay_ms_per_step": graph_ms,
+        "tile_plans": plans,
+        "wall_s_timed_region": wall,
+        "roofline": roof,
+    }
+    if unit == "TFLOP/s":
+        # time the whole step would take at max(matrix-core roof, HBM roof) of each product
+        ideal = sum(max(flops_one / (PEAK_BF16_TFLOPS * 1e12), abytes[p] / (PEAK_HBM_GBS * 1e9)) for p in per)
+        out["frac_of_step_roofline"] = ideal * 1e3 / ms_per_step
+    if sustained_seconds > 0:
+        # the same step for at least `sustained_seconds`: batches of `steps`, median and best batch
+        batches, t_end = [], time.perf_counter() + sustained_seconds
+        while time.perf_counter() < t_end or len(batches) < 3:
+            batches.append(_event_ms(step, steps, torch))
+        out["sustained"] = {"seconds": sustained_seconds, "batches": len(batches), "steps_per_batch": steps,
+                            "median_ms_per_step": statistics.median(batches), "min_ms_per_step": min(batches)}
+    if name == "decode":
+        out["bare_stream"] = bare_stream(copies, abytes["weights_read"], torch)
+    del x, A, dout, copies
+    torch.cuda.empty_cache()
+    return out
+
+
+def bare_stream(copies, nbytes, torch):
+    """A load-only kernel over as many bytes as the decode step streams (same rotation over weight copies), cut into
+    contiguous blocks of several sizes: the floor for a transfer this small on this box."""
+    from gpu_ragged_dot_amd import _capi
+
+    out = {}
+    stream = torch.cuda.current_stream().cuda_stream
+    for kib in (64, 128, 256, 352):
+        state = {"i": 0}
+
+        def read():
+            a = copies[state["i"] % len(copies)]
+            state["i"] += 1
+            _capi.check(_capi.lib.rd_probe_stream_read(stream, a.data_ptr(), nbytes, kib * 1024, None))
+
+        for _ in range(12):
+            read()
+        ms = _event_ms(read, 120, torch)
+        out["block_%dKiB" % kib] = {"us": ms * 1e3, "GB/s": nbytes / (ms * 1e-3) / 1e9}
+    return out
+
+
+def dense_gemm_context(torch):
+    """hipBLASLt (torch.matmul) on one dense bf16 GEMM with the Mixtral forward's FLOPs, on N(0,1) data and on zeros:
+    what the vendor library reaches on this box, and how much the data (power) matters."""
+    m, k, n = 16384, 4096, 14336
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    out = {}
+    for label in ("normal", "zeros"):
+        if label == "normal":
+            a = torch.randn((m, k), generator=gen, device="cuda").to(torch.bfloat16)
+            b = (torch.randn((k, n), generator=gen, device="cuda") / k ** 0.5).to(torch.bfloat16)
+        else:
+            a = torch.zeros((m, k), dtype=torch.bfloat16, device="cuda")
+            b = torch.zeros((k, n), dtype=torch.bfloat16, device="cuda")
+        c = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+        for _ in range(5):
+            torch.matmul(a, b, out=c)
+        ms = _event_ms(lambda: torch.matmul(a, b, out=c), 30, torch)
+        out[label] = {"ms": ms, "TFLOP/s": 2.0 * m * k * n / (ms * 1e-3) / 1e12}
+    return {"what": "torch.matmul bf16 [16384,4096]x[4096,14336] (the Mixtral forward's FLOPs as one dense GEMM)", **out}
+
+
 def bench_routing(args, torch):
     """The caller's side of the DeepSeek-V3 shaped workload: 4096 tokens x top-8 of 256 experts.  One step = route
     the (token, choice) pairs, gather the 7168-wide activations into expert order, and sum a 2048-wide product back
     per token.  HBM-bound byte work: reported as GB/s of algorithmic bytes (each tensor read or written once)."""
-    import numpy as np
-
     from gpu_ragged_dot_amd import moe
 
     tokens, top_k, g, d_in, d_out = 4096, 8, 256, 7168, 2048
@@ -152,9 +359,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="mixtral_fwd_bwd")
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD)
+    ap.add_argument("--only", action="store_true", help="measure the named workload only: no other configs, no context")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--cpu-seconds", type=float, default=6.0, help="CPU work per configuration for cpu_baseline")
+    ap.add_argument("--sustained-seconds", type=float, default=2.0)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy, so a counter run has a kernel of known traffic to scale by")
     args = ap.parse_args()
@@ -163,137 +372,49 @@ def main():
 
     import torch
 
-    import gpu_ragged_dot_amd as rd
-    from gpu_ragged_dot_amd import _capi, ops, planner, workloads
-
     name = args.workload
     if name == "moe_routing":
         return bench_routing(args, torch)
-    w = workloads.WORKLOADS[name]
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    x, A, dout, gs = workloads.make_inputs(name, device=dev)
-    hp = dict(block_m=64, block_k=64, block_n=64, interpret=False, compute_dtype=None, acc_dtype=torch.float32, chunk_m=512)
-
-    # For the memory-bound decode shape the 167 MB of expert weights would otherwise sit in the 256 MB last-level
-    # cache between steps: rotate over several copies so that every step streams from HBM.
-    copies = [A]
-    if name == "decode":
-        copies = [A] + [A.clone() for _ in range(5)]
-    state = {"i": 0}
-
-    def fwd():
-        a = copies[state["i"] % len(copies)]
-        state["i"] += 1
-        return ops._gmm_fwd(x, a, gs, **hp, trans_rhs=False)
-
-    def dlhs():
-        return ops._gmm_fwd(dout, A, gs, **hp, trans_rhs=True)
-
-    def drhs():
-        return ops._tgmm_fwd(x, dout, gs, **hp)
-
-    parts = [("fwd", fwd)] + ([("dlhs", dlhs), ("drhs", drhs)] if w.backward else [])
-
-    def step():
-        for _, fn in parts:
-            fn()
+    torch.cuda.set_device(0)
+    full = not args.only and name == DEFAULT_WORKLOAD and not args.copy_calibration
 
     if args.copy_calibration:
-        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
         dst = torch.empty_like(src)
         for _ in range(3):
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    ms_per_step = _event_ms(step, args.steps, torch)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-
-    # The decode step is one ~40 us launch: also time it replayed from a HIP graph (one graph = one call per weight
-    # copy), which takes the host's launch path out of the measurement.
-    graph_ms = None
-    if name == "decode":
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            for a in copies:
-                ops._gmm_fwd(x, a, gs, **hp, trans_rhs=False)
-        for _ in range(3):
-            graph.replay()
-        graph_ms = _event_ms(graph.replay, max(args.steps // len(copies), 4), torch) / len(copies)
-
-    # per-kernel launch durations, for the roofline of the dominant kernel
-    if len(parts) == 1:  # the step is that one product: the timed region already is its launch duration
-        per = {parts[0][0]: ms_per_step}
-    else:
-        per = {pname: _event_ms(fn, max(args.steps, 5), torch) for pname, fn in parts}
-    dominant = max(per, key=per.get)
-    flops_step = workloads.flops(name)
-    abytes = workloads.algorithmic_bytes(name)
-    flops_one = flops_step / (3 if w.backward else 1)
-
-    if name == "decode":
-        metric, unit = "ragged_dot decode forward, expert weights streamed", "GB/s"
-        value = abytes["weights_read"] / (ms_per_step * 1e-3) / 1e9
-        roof = {"bound": "hbm", "achieved": abytes[dominant] / (per[dominant] * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
-                "unit": "GB/s"}
-    else:
-        metric, unit = ("ragged_dot fwd+bwd" if w.backward else "ragged_dot fwd") + " throughput", "TFLOP/s"
-        value = flops_step / (ms_per_step * 1e-3) / 1e12
-        t_flop = flops_one / (PEAK_BF16_TFLOPS * 1e12)
-        t_byte = abytes[dominant] / (PEAK_HBM_GBS * 1e9)
-        if t_byte > t_flop:
-            roof = {"bound": "hbm", "achieved": abytes[dominant] / (per[dominant] * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
-                    "unit": "GB/s"}
-        else:
-            roof = {"bound": "mfma", "achieved": flops_one / (per[dominant] * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
-                    "unit": "TFLOP/s"}
-    roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = None  # HBM bytes per launch of the dominant kernel, from committed counter runs (profiles/)
-    try:
-        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
-            roof["traffic"] = json.load(f).get(name, {}).get(dominant)
-    except (OSError, ValueError):
-        pass
-    roof["kernel"] = {"fwd": "gmm_kernel<.., trans_rhs=false>" if name != "decode" else "gmm_rows_kernel + gmm_rows_finish_kernel",
-                      "dlhs": "gmm_kernel<.., trans_rhs=true>", "drhs": "tgmm_kernel"}[dominant]
-    roof["launch_ms"] = per[dominant]
-
-    plans = {}
-    for pname, op, (mm, kk, nn) in (("fwd", 0, (w.m, w.k, w.n)), ("dlhs", 1, (w.m, w.n, w.k)), ("drhs", 2, (w.m, w.k, w.n))):
-        if pname in per:
-            p = planner.select_plan(op, mm, kk, nn, w.g)
-            plans[pname] = ("decode_rows" if p.decode_nb < 0 else "decode_nb%d" % p.decode_nb) if p.decode_nb else planner.compiled_variants()[p.variant].name.decode()
-
+    head = measure(name, args.steps, args.warmup, torch, sustained_seconds=args.sustained_seconds if full else 0.0, headline=True)
     out = {
-        "metric": metric,
-        "value": value,
-        "unit": unit,
+        "metric": head.pop("metric"),
+        "value": head.pop("value"),
+        "unit": head.pop("unit"),
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
+        "steps": head.pop("steps"),
+        "warmup": head.pop("warmup"),
+        "ms_per_step": head.pop("ms_per_step"),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": name, "m": w.m, "k": w.k, "n": w.n, "g": w.g, "backward": w.backward,
-                   "description": w.description, "group_sizes": "seeded, see gpu_ragged_dot_amd/workloads.py"},
-        "frac_of_bf16_mfma_peak": (value / PEAK_BF16_TFLOPS) if unit == "TFLOP/s" else None,
-        "per_kernel_ms": per,
-        "graph_replay_ms_per_step": graph_ms,
-        "tile_plans": plans,
-        "wall_s_timed_region": wall,
-        "roofline": roof,
     }
+    out.update(head)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(name, args.cpu_seconds)
+    if full:
+        configs = {}
+        for other in OTHER_CONFIGS:
+            c = measure(other, args.steps, args.warmup, torch)
+            if not args.no_cpu_baseline:
+                c["cpu_baseline"] = cpu_baseline(other, args.cpu_seconds)
+            configs[other] = c
+        out["configs"] = configs
+        out["context"] = {"dense_gemm": dense_gemm_context(torch), "sustained_headline_step": out.pop("sustained", None),
+                          "decode_bare_stream": configs["decode"].pop("bare_stream", None), "cpu": cpu_model(),
+                          "device": torch.cuda.get_device_name(0)}
     print(json.dumps(out))
 
 

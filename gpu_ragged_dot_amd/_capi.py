@@ -85,6 +85,7 @@ EXPORTS = (
     "rd_gmm_noalloc",
     "rd_tgmm_workspace_bytes",
     "rd_tgmm",
+    "rd_probe_stream_read",
     "rd_moe_route_workspace_bytes",
     "rd_moe_route",
     "rd_moe_dispatch",
@@ -129,6 +130,8 @@ def _load() -> ctypes.CDLL:
     lib.rd_tgmm_workspace_bytes.restype = sz
     lib.rd_tgmm.argtypes = [vp, vp, vp, ip, vp, i, i, i, i, i, ctypes.POINTER(Plan), vp, sz]
     lib.rd_tgmm.restype = i
+    lib.rd_probe_stream_read.argtypes = [vp, vp, sz, sz, vp]
+    lib.rd_probe_stream_read.restype = i
     lib.rd_moe_route_workspace_bytes.argtypes = [i, i, i]
     lib.rd_moe_route_workspace_bytes.restype = sz
     lib.rd_moe_route.argtypes = [vp, ip, i, i, i, ip, ip, ip, vp, sz]

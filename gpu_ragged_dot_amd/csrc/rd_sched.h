@@ -18,6 +18,9 @@ int launch_sched_map(hipStream_t s, const int32_t* group_sizes, int g, int m, in
                      int32_t* tile2group, int32_t* tile2it, int32_t* total_tiles, int32_t* counters = nullptr,
                      int n_counters = 0, int32_t* tile2band = nullptr, int band_rows = 1);
 
+// Measurement aid: a bare read of `bytes` (16-byte aligned) cut into contiguous blocks of block_bytes, one work-group each.
+int launch_stream_read(hipStream_t s, const void* src, size_t bytes, size_t block_bytes, void* sink);
+
 // Stream-ordered clear that is safe to record into a HIP graph.
 int launch_zero_bytes(hipStream_t s, void* p, size_t bytes);
 

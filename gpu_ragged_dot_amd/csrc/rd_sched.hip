@@ -107,7 +107,35 @@ __global__ void fill_kernel(T* p, size_t n, T v) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
 }
 
+// Load-only kernel: work-group b reads block b (block_bytes contiguous bytes, the last one shorter) with streaming
+// 16-byte loads and folds what it read into one word that is stored only if it equals a value the caller never expects,
+// which keeps the loads alive without a store stream.
+__global__ __launch_bounds__(256) void stream_read_kernel(const u32x4_t* __restrict__ src, size_t n16, size_t block16,
+                                                          uint32_t* __restrict__ sink, uint32_t never) {
+  const size_t lo = (size_t)blockIdx.x * block16, hi = lo + block16 < n16 ? lo + block16 : n16;
+  u32x4_t acc = {0, 0, 0, 0};
+  size_t i = lo + threadIdx.x;
+  for (; i + 3 * 256 < hi; i += 4 * 256) {  // four independent loads in flight per thread
+    const u32x4_t a = __builtin_nontemporal_load(src + i), b = __builtin_nontemporal_load(src + i + 256);
+    const u32x4_t c = __builtin_nontemporal_load(src + i + 512), d = __builtin_nontemporal_load(src + i + 768);
+    acc ^= a ^ b ^ c ^ d;
+  }
+  for (; i < hi; i += 256) acc ^= __builtin_nontemporal_load(src + i);
+  const uint32_t w = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+  if (w == never && sink) *sink = w;
+}
+
 }  // namespace
+
+int launch_stream_read(hipStream_t s, const void* src, size_t bytes, size_t block_bytes, void* sink) {
+  const size_t n16 = bytes / 16, block16 = block_bytes / 16;
+  if (n16 == 0 || block16 == 0) return hipSuccess;
+  const size_t blocks = (n16 + block16 - 1) / block16;
+  if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(stream_read_kernel, dim3((unsigned)blocks), dim3(256), 0, s, static_cast<const u32x4_t*>(src), n16, block16,
+                     static_cast<uint32_t*>(sink), 0x9e3779b9u);
+  return (int)hipGetLastError();
+}
 
 int launch_sched_map(hipStream_t s, const int32_t* gs, int g, int m, int chunk, int32_t* group_offsets,
                      int32_t* tile2group, int32_t* tile2it, int32_t* total_tiles, int32_t* counters, int n_counters,

@@ -49,7 +49,9 @@ def sweep(x, A, dout, gs, op: int, reps: int = 10, rounds: int = 3):
     g = A.shape[0]
     n = A.shape[2]
     vec = k % 8 == 0 and n % 8 == 0
-    walks = [(0, 0), (2, 4), (4, 4), (8, 4), (2, 8), (4, 8)] if op != _capi.OP_TGMM else [(4, 0), (8, 0), (16, 0)]
+    # gmm: (most row tiles per band, columns per block); the product is what one XCD is dealt at a time, 32 tiles suit
+    # one work-group per compute unit.  tgmm: row tiles per band.
+    walks = [(0, 0), (1, 32), (2, 16), (4, 8), (8, 4), (2, 4), (4, 4)] if op != _capi.OP_TGMM else [(1, 0), (2, 0), (4, 0), (8, 0), (16, 0)]
     cands = []
     for v in planner.compiled_variants():
         if bool(v.vec) != vec or v.dtype != _capi.RD_DTYPE_BF16:

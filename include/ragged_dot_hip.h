@@ -126,6 +126,13 @@ int rd_tgmm(void* stream, const void* x, const void* dy, const int32_t* group_si
             int n, int g, int dtype, const rd_plan* plan /* host, may be NULL */, void* workspace,
             size_t workspace_bytes);
 
+/* ---- measurement aid ----------------------------------------------------------------------------------------------
+ * No counterpart in the reference.  A load-only kernel: reads `bytes` (src 16-byte aligned) cut into contiguous blocks
+ * of block_bytes, one work-group per block, and stores nothing (`sink`, 4 bytes of device memory or NULL, is written
+ * only if the folded data equals one fixed word).  It is what a bare stream over the same bytes takes on this device -
+ * the floor the benchmark prints next to the memory-bound kernels. */
+int rd_probe_stream_read(void* stream, const void* src, size_t bytes, size_t block_bytes, void* sink);
+
 /* ---- token routing around ragged_dot --------------------------------------------------------------------------
  * The reference takes rows that are already sorted by group and leaves the sorting to its caller (its tests and
  * tuner build sorted rows directly: tests.py:51-71, tuning.py:41-47).  These entry points are that caller's side for a
