@@ -76,13 +76,11 @@ __device__ __forceinline__ void run_tile(const typename C::Elem* Ap, int lda, in
 // tall tiles of long groups share.
 // A 128-row routine of the same kind (6 slabs of 32, or 3 of 64) serves the tiles with 65 to 128 rows.
 constexpr int kShortRows = 64, kMidRows = 128;
-// STREAM: the group has this one row tile only, so nobody else reads its weights.  The short last tile of a longer
-// group runs the same routine with the default cache policy: its band's other tiles read the same weights from L2.
-template <class C, int ROWS, bool STREAM>
+template <class C, int ROWS>
 struct ShortTileCfg {
   static constexpr int BK = C::B_KMAJOR ? 64 : 32;
   static constexpr int STAGES = (160 * 1024) / ((ROWS + C::BN) * BK * 2);
-  typedef DldsCfg<ROWS, C::BN, BK, 1, 4, true, C::B_KMAJOR, STAGES, false, STREAM ? kCachePolicyStream : 0> type;
+  typedef DldsCfg<ROWS, C::BN, BK, 1, 4, true, C::B_KMAJOR, STAGES, false, kCachePolicyStream> type;
 };
 
 // How the last round of a gmm launch is cut along K.  The device runs num_cus tiles at a time; when the live tiles do
@@ -202,22 +200,17 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
                             : pA + (size_t)gi * p.k * p.n + (size_t)k0 * p.n + col0;
     E* Op = py + (size_t)row0 * p.n + col0;
     if constexpr (IsW4<C>::value && C::A_KMAJOR) {
-      if (rows <= kMidRows) {
-        typedef typename ShortTileCfg<C, kShortRows, true>::type S;
-        typedef typename ShortTileCfg<C, kMidRows, true>::type M;
-        typedef typename ShortTileCfg<C, kShortRows, false>::type SL;
-        typedef typename ShortTileCfg<C, kMidRows, false>::type ML;
+      // Only for a group's single row tile.  The short last tile of a longer group stays on the tall routine: run
+      // through the short one it finishes early, the tiles dealt next start out of step with the rest of their block,
+      // and the block's operand slabs are fetched into L2 twice (measured: +1 GB of fetches per launch, no time gained).
+      if (rows <= kMidRows && it == 0) {
+        typedef typename ShortTileCfg<C, kShortRows>::type S;
+        typedef typename ShortTileCfg<C, kMidRows>::type M;
         static_assert(S::LDS_BYTES <= C::LDS_BYTES && S::NT == C::NT && S::BN == C::BN, "the short routine runs in the tall one's launch");
         static_assert(M::LDS_BYTES <= C::LDS_BYTES && M::NT == C::NT && M::BN == C::BN, "the 128-row routine runs in the tall one's launch");
         const int ldb = TRANS_RHS ? p.k : p.n;
-        const bool only_tile = it == 0;  // rows <= 128 and first tile: the group has no other
-        if (rows <= kShortRows) {
-          if (only_tile) gemm_tile_dlds<S>(Ap, p.k, rows, Bp, ldb, cols, klen, Op, p.n, smem, sk);
-          else gemm_tile_dlds<SL>(Ap, p.k, rows, Bp, ldb, cols, klen, Op, p.n, smem, sk);
-        } else {
-          if (only_tile) gemm_tile_dlds<M>(Ap, p.k, rows, Bp, ldb, cols, klen, Op, p.n, smem, sk);
-          else gemm_tile_dlds<ML>(Ap, p.k, rows, Bp, ldb, cols, klen, Op, p.n, smem, sk);
-        }
+        if (rows <= kShortRows) gemm_tile_dlds<S>(Ap, p.k, rows, Bp, ldb, cols, klen, Op, p.n, smem, sk);
+        else gemm_tile_dlds<M>(Ap, p.k, rows, Bp, ldb, cols, klen, Op, p.n, smem, sk);
         return;
       }
     }
