@@ -159,3 +159,25 @@ def test_cpu_tensors_are_rejected_loudly():
         rd.ragged_dot(x, A, torch.tensor([4, 2, 2], dtype=torch.int32))  # gpu_ragged_dot.py:189
     with pytest.raises(AssertionError):
         rd.tgmm(x, torch.zeros(9, 8, dtype=torch.bfloat16), torch.tensor([4, 4], dtype=torch.int32))  # :304
+
+
+def test_committed_traffic_figures_belong_to_the_plans_in_use():
+    """profiles/hbm_traffic.json tags every counter-derived figure with the plan it was measured under; bench.py drops a
+    figure whose tag is not the plan in use.  Keep the committed table in step with the planner."""
+    import json
+    import os
+
+    import bench
+    from gpu_ragged_dot_amd import workloads
+
+    with open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "profiles", "hbm_traffic.json")) as f:
+        table = json.load(f)
+    for name, kernels in table.items():
+        if name.startswith("_"):
+            continue
+        w = workloads.WORKLOADS[name]
+        dims = {"fwd": (0, w.m, w.k, w.n), "dlhs": (1, w.m, w.n, w.k), "drhs": (2, w.m, w.k, w.n)}
+        for kernel, entry in kernels.items():
+            op, m, k, n = dims[kernel]
+            assert entry["bytes"] > 0
+            assert entry["plan"] == bench._plan_text(planner.select_plan(op, m, k, n, w.g), planner), (name, kernel)
