@@ -81,6 +81,8 @@ EXPORTS = (
     "rd_sched_map_len",
     "rd_gmm_workspace_bytes",
     "rd_gmm",
+    "rd_gmm_sharded",
+    "rd_tgmm_sharded",
     "rd_gmm_noalloc_scratch_bytes",
     "rd_gmm_noalloc",
     "rd_tgmm_workspace_bytes",
@@ -122,6 +124,10 @@ def _load() -> ctypes.CDLL:
     lib.rd_gmm_workspace_bytes.restype = sz
     lib.rd_gmm.argtypes = [vp, vp, vp, ip, vp, i, i, i, i, i, i, ctypes.POINTER(Plan), vp, sz]
     lib.rd_gmm.restype = i
+    lib.rd_gmm_sharded.argtypes = [vp, vp, vp, ip, vp, i, i, i, i, i, i, i, i, ctypes.POINTER(Plan), vp, sz]
+    lib.rd_gmm_sharded.restype = i
+    lib.rd_tgmm_sharded.argtypes = [vp, vp, vp, ip, vp, i, i, i, i, i, i, i, ctypes.POINTER(Plan), vp, sz]
+    lib.rd_tgmm_sharded.restype = i
     lib.rd_gmm_noalloc_scratch_bytes.argtypes = []
     lib.rd_gmm_noalloc_scratch_bytes.restype = sz
     lib.rd_gmm_noalloc.argtypes = [vp, vp, vp, ip, vp, i, i, i, i, i, i, ctypes.POINTER(Plan)]

@@ -21,7 +21,8 @@ struct GmmArgs {
   const int32_t* tile2it;        // [U]
   const int32_t* tile2band;      // [U]   band of row tiles each row tile belongs to (see rd_sched.h)
   const int32_t* total_tiles;    // [1]
-  int m, k, n, g;
+  int m, k, n, g;  // g: all groups of group_sizes
+  int g_first, g_local;  // A holds the g_local groups [g_first, g_first + g_local); rows of the others are zero
   int U;        // static bound on row tiles: ceil(m / BM) + g
   int n_tiles;  // ceil(n / BN)
   int group_m, group_n;  // tile walk: most row tiles per band; positions per block = group_m x group_n
@@ -41,7 +42,8 @@ struct TgmmArgs {
   void* dA;
   const int32_t* group_sizes;
   const int32_t* group_offsets;
-  int m, k, n, g;
+  int m, k, n, g;  // g: groups of dA (the slices computed)
+  int g_first;     // dA[i] belongs to group g_first + i of group_sizes / group_offsets
   int k_tiles, n_tiles;  // ceil(k / BM), ceil(n / BN)
   int group_m;
 };
@@ -195,10 +197,16 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
     int rows = imin(C::BM, uniform(p.group_sizes[gi]) - it * C::BM);
     rows = imin(rows, p.m - row0);  // group_sizes summing past m: never touch rows >= m
     if (rows <= 0 || row0 < 0) return;
-    const E* Ap = px + (size_t)row0 * p.k + k0;
-    const E* Bp = TRANS_RHS ? pA + (size_t)gi * p.n * p.k + (size_t)col0 * p.k + k0
-                            : pA + (size_t)gi * p.k * p.n + (size_t)k0 * p.n + col0;
     E* Op = py + (size_t)row0 * p.n + col0;
+    const int gl = gi - p.g_first;  // index of the group's weights in A
+    if (gl < 0 || gl >= p.g_local) {
+      // a group whose weights live elsewhere (A is a slice of the groups): its rows of y are zero
+      if (sk.part == 0) zero_tile<C::NT, C::VEC, E>(Op, p.n, rows, cols);
+      return;
+    }
+    const E* Ap = px + (size_t)row0 * p.k + k0;
+    const E* Bp = TRANS_RHS ? pA + (size_t)gl * p.n * p.k + (size_t)col0 * p.k + k0
+                            : pA + (size_t)gl * p.k * p.n + (size_t)k0 * p.n + col0;
     if constexpr (IsW4<C>::value && C::A_KMAJOR) {
       // Only for a group's single row tile.  The short last tile of a longer group stays on the tall routine: run
       // through the short one it finishes early, the tiles dealt next start out of step with the rest of their block,
@@ -249,8 +257,8 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void tgmm_kernel(TgmmArgs p
   const int krows = imin(C::BM, p.k - kk0), cols = imin(C::BN, p.n - col0);
   E* Op = static_cast<E*>(p.dA) + (size_t)gi * p.k * p.n + (size_t)kk0 * p.n + col0;
 
-  const int row0 = uniform(p.group_offsets[gi]);
-  int rows = uniform(p.group_sizes[gi]);
+  const int row0 = uniform(p.group_offsets[gi + p.g_first]);
+  int rows = uniform(p.group_sizes[gi + p.g_first]);
   rows = imin(rows, p.m - row0);
   if (rows <= 0 || row0 < 0) {  // empty group: its slice of dA is zero
     zero_tile<C::NT, C::VEC, E>(Op, p.n, krows, cols);

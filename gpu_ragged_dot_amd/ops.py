@@ -71,16 +71,34 @@ def _plan_ref(plan: Optional[_capi.Plan]):
     return ctypes.byref(plan) if plan is not None else None
 
 
+def _group_offset(group_offset) -> int:
+    """``group_offset`` as a host integer (None = 0; a one-element tensor is read back, which synchronises)."""
+    if group_offset is None:
+        return 0
+    if isinstance(group_offset, torch.Tensor):
+        assert group_offset.numel() == 1, "group_offset holds one group index"
+        return int(group_offset.item())
+    return int(group_offset)
+
+
 def _gmm_fwd(x, A, group_sizes, block_m, block_k, block_n, trans_rhs, interpret, compute_dtype, acc_dtype, chunk_m,
-             plan: Optional[_capi.Plan] = None) -> torch.Tensor:
-    """gpu_ragged_dot.py:171-228 (_gpu_gmm_fwd): checks, planning, one call across the C ABI."""
+             plan: Optional[_capi.Plan] = None, group_offset=None) -> torch.Tensor:
+    """gpu_ragged_dot.py:171-228 (_gpu_gmm_fwd): checks, planning, one call across the C ABI.
+
+    ``group_offset`` (jax.lax.ragged_dot's parameter; not in the reference): A holds the groups
+    [group_offset, group_offset + A.shape[0]) of the ones group_sizes describes; rows of the others come out zero."""
     if interpret:
         raise NotImplementedError("interpret=True (Pallas interpreter) has no counterpart; kernels run on the GPU only")
     assert A.ndim == 3 and x.ndim == 2, f"but {A.ndim=} {x.ndim=}"  # :188
     gs_host_shape = tuple(torch.as_tensor(group_sizes).shape)
-    assert tuple(A.shape[:1]) == gs_host_shape, f"{A.shape[:1]=} != {gs_host_shape=}"  # :189
+    g_first = _group_offset(group_offset)
+    if group_offset is None:
+        assert tuple(A.shape[:1]) == gs_host_shape, f"{A.shape[:1]=} != {gs_host_shape=}"  # :189
+    else:
+        assert len(gs_host_shape) == 1 and 0 <= g_first and g_first + A.shape[0] <= gs_host_shape[0], \
+            f"groups [{g_first}, {g_first}+{A.shape[0]}) are not within {gs_host_shape=}"
     m, k = x.shape
-    g = A.shape[0]
+    g_local, g = A.shape[0], gs_host_shape[0]
     n = A.shape[-1] if not trans_rhs else A.shape[-2]  # :190
     k_rhs = A.shape[-2] if not trans_rhs else A.shape[-1]
     assert k_rhs == k, f"contraction mismatch: x has k={k}, A has {k_rhs}"
@@ -96,19 +114,23 @@ def _gmm_fwd(x, A, group_sizes, block_m, block_k, block_n, trans_rhs, interpret,
     if plan is None:
         plan = planner.select_plan(_capi.OP_GMM_TRANS if trans_rhs else _capi.OP_GMM, m, k, n, g, block_m, block_k, block_n,
                                    dtype=code, aligned=_aligned16(x, A, y))
+    if (g_first, g_local) != (0, g) and plan.decode_nb:
+        plan = _capi.Plan(plan.variant, plan.group_m, 0, plan.group_n, plan.split_k)  # streaming kernels: all groups only
     ws_bytes = _capi.lib.rd_gmm_workspace_bytes(m, g, _plan_ref(plan))
     ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         _capi.check(
-            _capi.lib.rd_gmm(_stream_ptr(dev), x.data_ptr(), A.data_ptr(), gs.data_ptr(), y.data_ptr(), m, k, n, g,
-                             int(bool(trans_rhs)), code, _plan_ref(plan), ws.data_ptr(), ws.numel())
+            _capi.lib.rd_gmm_sharded(_stream_ptr(dev), x.data_ptr(), A.data_ptr(), gs.data_ptr(), y.data_ptr(), m, k, n,
+                                     g, g_first, g_local, int(bool(trans_rhs)), code, _plan_ref(plan), ws.data_ptr(),
+                                     ws.numel())
         )
     return y
 
 
 def _tgmm_fwd(x, y, group_sizes, block_m, block_k, block_n, interpret, compute_dtype, acc_dtype, chunk_m,
-              plan: Optional[_capi.Plan] = None) -> torch.Tensor:
-    """gpu_ragged_dot.py:287-342 (_gpu_tgmm_fwd)."""
+              plan: Optional[_capi.Plan] = None, group_offset=None, num_actual_groups=None) -> torch.Tensor:
+    """gpu_ragged_dot.py:287-342 (_gpu_tgmm_fwd).  With ``group_offset`` / ``num_actual_groups`` only the slices of the
+    groups [group_offset, group_offset + num_actual_groups) are computed: out[i] belongs to group group_offset + i."""
     del chunk_m  # :303
     if interpret:
         raise NotImplementedError("interpret=True (Pallas interpreter) has no counterpart; kernels run on the GPU only")
@@ -123,7 +145,10 @@ def _tgmm_fwd(x, y, group_sizes, block_m, block_k, block_n, interpret, compute_d
         raise TypeError(f"x is {x.dtype} but y is {y.dtype}")
     x, y = x.contiguous(), y.contiguous()
     gs = _group_sizes_i32(gs_t, dev)
-    out = torch.empty((g, k, n), dtype=x.dtype, device=dev)  # :324
+    g_first = _group_offset(group_offset)
+    g_local = g - g_first if num_actual_groups is None else int(num_actual_groups)
+    assert 0 <= g_first and g_local >= 1 and g_first + g_local <= g, f"groups [{g_first}, {g_first}+{g_local}) are not within {g}"
+    out = torch.empty((g_local, k, n), dtype=x.dtype, device=dev)  # :324
     if plan is None:
         plan = planner.select_plan(_capi.OP_TGMM, m, k, n, g, block_m, block_k, block_n, dtype=code,
                                    aligned=_aligned16(x, y, out))
@@ -131,8 +156,8 @@ def _tgmm_fwd(x, y, group_sizes, block_m, block_k, block_n, interpret, compute_d
     ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         _capi.check(
-            _capi.lib.rd_tgmm(_stream_ptr(dev), x.data_ptr(), y.data_ptr(), gs.data_ptr(), out.data_ptr(), m, k, n, g,
-                              code, _plan_ref(plan), ws.data_ptr(), ws.numel())
+            _capi.lib.rd_tgmm_sharded(_stream_ptr(dev), x.data_ptr(), y.data_ptr(), gs.data_ptr(), out.data_ptr(), m, k, n,
+                                      g, g_first, g_local, code, _plan_ref(plan), ws.data_ptr(), ws.numel())
         )
     return out
 
@@ -155,9 +180,10 @@ class _GmmFn(torch.autograd.Function):
         do = do.contiguous()
         dx = dA = None
         if ctx.needs_input_grad[0]:
-            dx = _gmm_fwd(do, A, group_sizes, **hp, trans_rhs=not trans_rhs)  # :400
+            dx = _gmm_fwd(do, A, group_sizes, **hp, trans_rhs=not trans_rhs)  # :400 (rows of groups outside A's slice: zero)
         if ctx.needs_input_grad[1]:
             thp = {k_: v for k_, v in hp.items()}
+            thp["num_actual_groups"] = A.shape[0]
             dA = _tgmm_fwd(x, do, group_sizes, **thp) if not trans_rhs else _tgmm_fwd(do, x, group_sizes, **thp)  # :401
         return dx, dA, None, None  # group_sizes gets no cotangent, :402
 
@@ -176,6 +202,7 @@ class _TgmmFn(torch.autograd.Function):
         x, y, group_sizes = ctx.saved_tensors
         hp = dict(ctx.hp)
         hp.pop("plan", None)
+        hp.pop("num_actual_groups", None)  # do has that many slices; group_offset says which groups they are
         do = do.contiguous()
         dx = dy = None
         if ctx.needs_input_grad[0]:
@@ -199,15 +226,20 @@ def gmm(
     num_warps: Optional[int] = None,
     num_stages: Optional[int] = None,
     chunk_m: int = CHUNK_M,
+    group_offset=None,
 ) -> torch.Tensor:
     """Ragged dot corresponding to jax.lax.ragged_dot: (m, k) x (g, k, n) -> (m, n).  gpu_ragged_dot.py:362-380.
 
     ``num_warps`` / ``num_stages`` are Triton knobs of the reference and are accepted and ignored; ``chunk_m`` is
-    validated only (the kernels split groups by their own tile height).
+    validated only (the kernels split groups by their own tile height).  ``group_offset`` (after the reference's
+    parameters; jax.lax.ragged_dot's own keyword): A holds only the groups [group_offset, group_offset + A.shape[0])
+    of those in group_sizes - an expert-parallel rank's slice; rows of the other groups are zero.
     """
     del num_warps, num_stages
     hp = dict(block_m=block_m, block_k=block_k, block_n=block_n, trans_rhs=trans_rhs, interpret=interpret,
               compute_dtype=compute_dtype, acc_dtype=acc_dtype, chunk_m=chunk_m)
+    if group_offset is not None:
+        hp["group_offset"] = _group_offset(group_offset)
     if torch.is_grad_enabled() and (x.requires_grad or A.requires_grad):
         gs = _group_sizes_i32(group_sizes, x.device)
         return _GmmFn.apply(x, A, gs, hp)
@@ -227,11 +259,17 @@ def tgmm(
     num_warps: Optional[int] = None,
     num_stages: Optional[int] = None,
     chunk_m: int = CHUNK_M,
+    group_offset=None,
+    num_actual_groups: Optional[int] = None,
 ) -> torch.Tensor:
-    """Transposed ragged dot: (m, k) x (m, n) -> (g, k, n).  gpu_ragged_dot.py:411-428."""
+    """Transposed ragged dot: (m, k) x (m, n) -> (g, k, n).  gpu_ragged_dot.py:411-428.  With ``group_offset`` /
+    ``num_actual_groups`` only the slices of the groups [group_offset, group_offset + num_actual_groups) are computed."""
     del num_warps, num_stages
     hp = dict(block_m=block_m, block_k=block_k, block_n=block_n, interpret=interpret, compute_dtype=compute_dtype,
               acc_dtype=acc_dtype, chunk_m=chunk_m)
+    if group_offset is not None or num_actual_groups is not None:
+        hp["group_offset"] = _group_offset(group_offset)
+        hp["num_actual_groups"] = num_actual_groups
     if torch.is_grad_enabled() and (x.requires_grad or y.requires_grad):
         gs = _group_sizes_i32(group_sizes, x.device)
         return _TgmmFn.apply(x, y, gs, hp)

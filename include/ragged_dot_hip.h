@@ -105,6 +105,22 @@ int rd_gmm(void* stream, const void* x, const void* A, const int32_t* group_size
            int g, int trans_rhs, int dtype, const rd_plan* plan /* host, may be NULL */, void* workspace,
            size_t workspace_bytes);
 
+/* ---- a slice of the groups (expert-parallel sharding) ----------------------------------------------------------
+ * The `group_offset` of jax.lax.ragged_dot (named by its documentation; the reference gpu_ragged_dot.py has no such
+ * parameter).  group_sizes still describes all g_total groups and x / y all m rows, but A (dA) holds only the
+ * g_local groups [group_offset, group_offset + g_local): a rank that owns a slice of the experts calls with its
+ * slice and the global group_sizes.
+ *   rd_gmm_sharded : rows of the groups in the slice as rd_gmm; rows of every other group and past sum(group_sizes) zero.
+ *   rd_tgmm_sharded: dA[i] = slice of group group_offset + i, i < g_local.
+ * Workspace: rd_gmm_workspace_bytes / rd_tgmm_workspace_bytes with g = g_total.  The streaming kernels
+ * (plan.decode_nb != 0) serve all groups only.  group_offset = 0 and g_local = g_total is rd_gmm / rd_tgmm. */
+int rd_gmm_sharded(void* stream, const void* x, const void* A, const int32_t* group_sizes, void* y, int m, int k, int n,
+                   int g_total, int group_offset, int g_local, int trans_rhs, int dtype,
+                   const rd_plan* plan /* host, may be NULL */, void* workspace, size_t workspace_bytes);
+int rd_tgmm_sharded(void* stream, const void* x, const void* dy, const int32_t* group_sizes, void* dA, int m, int k, int n,
+                    int g_total, int group_offset, int g_local, int dtype, const rd_plan* plan /* host, may be NULL */,
+                    void* workspace, size_t workspace_bytes);
+
 /* ---- rd_gmm without a workspace -------------------------------------------------------------------------------
  * No counterpart in the reference.  For callers that cannot allocate device memory: code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc.  Same product as rd_gmm, same kernels; what rd_gmm keeps in the

@@ -152,10 +152,13 @@ def _offsets(group_sizes: np.ndarray) -> np.ndarray:
     return np.concatenate([[0], np.cumsum(gs)])
 
 
-def gmm(x, A, group_sizes, trans_rhs: bool = False, out_dtype: str = "bfloat16", acc=np.float32) -> np.ndarray:
+def gmm(x, A, group_sizes, trans_rhs: bool = False, out_dtype: str = "bfloat16", acc=np.float32,
+        group_offset: int = 0) -> np.ndarray:
     """y[rows of group g] = x[rows] @ A[g] (or @ A[g].T), rows >= sum(group_sizes) are zero.
 
     gpu_ragged_dot.py:108-150 (which rows a work item owns; dtype flow :116-119,145-149) and :155-165 (tail zero).
+    group_offset (jax.lax.ragged_dot's keyword, not in the reference): A[i] are the weights of group group_offset + i;
+    rows of the groups A does not hold are zero.  Pinned by: the product with the missing groups' weights set to zero.
     """
     x = np.asarray(x, dtype=acc)
     A = np.asarray(A, dtype=acc)
@@ -164,19 +167,22 @@ def gmm(x, A, group_sizes, trans_rhs: bool = False, out_dtype: str = "bfloat16",
     off = _offsets(group_sizes)
     y = np.zeros((m, n), dtype=acc)
     for gi in range(A.shape[0]):
-        lo, hi = min(int(off[gi]), m), min(int(off[gi + 1]), m)
+        lo, hi = min(int(off[gi + group_offset]), m), min(int(off[gi + group_offset + 1]), m)
         if hi > lo:
             y[lo:hi] = x[lo:hi] @ (A[gi].T if trans_rhs else A[gi])
     return round_to(y, out_dtype) if acc == np.float32 else y
 
 
-def tgmm(x, y, group_sizes, out_dtype: str = "bfloat16", acc=np.float32) -> np.ndarray:
-    """A_bar[g] = x[rows of g].T @ y[rows of g]; empty group -> zeros (gpu_ragged_dot.py:250-281)."""
+def tgmm(x, y, group_sizes, out_dtype: str = "bfloat16", acc=np.float32, group_offset: int = 0,
+         num_actual_groups=None) -> np.ndarray:
+    """A_bar[g] = x[rows of g].T @ y[rows of g]; empty group -> zeros (gpu_ragged_dot.py:250-281).  With group_offset /
+    num_actual_groups: only the slices of the groups [group_offset, group_offset + num_actual_groups)."""
     x = np.asarray(x, dtype=acc)
     y = np.asarray(y, dtype=acc)
     m = x.shape[0]
     off = _offsets(group_sizes)
-    g = len(off) - 1
+    g = (len(off) - 1 - group_offset) if num_actual_groups is None else int(num_actual_groups)
+    off = off[group_offset:]
     out = np.zeros((g, x.shape[1], y.shape[1]), dtype=acc)
     for gi in range(g):
         lo, hi = min(int(off[gi]), m), min(int(off[gi + 1]), m)
@@ -185,13 +191,15 @@ def tgmm(x, y, group_sizes, out_dtype: str = "bfloat16", acc=np.float32) -> np.n
     return round_to(out, out_dtype) if acc == np.float32 else out
 
 
-def gmm_vjp(x, A, group_sizes, dout, trans_rhs: bool = False, out_dtype: str = "bfloat16", acc=np.float32):
+def gmm_vjp(x, A, group_sizes, dout, trans_rhs: bool = False, out_dtype: str = "bfloat16", acc=np.float32,
+            group_offset: int = 0):
     """gpu_ragged_dot.py:383-402: dx = gmm(do, A, !trans_rhs); dA = tgmm(x, do) or tgmm(do, x); None for sizes."""
-    dx = gmm(dout, A, group_sizes, trans_rhs=not trans_rhs, out_dtype=out_dtype, acc=acc)  # :400
+    kw = dict(out_dtype=out_dtype, acc=acc, group_offset=group_offset)
+    dx = gmm(dout, A, group_sizes, trans_rhs=not trans_rhs, **kw)  # :400
     if not trans_rhs:
-        dA = tgmm(x, dout, group_sizes, out_dtype=out_dtype, acc=acc)  # :401
+        dA = tgmm(x, dout, group_sizes, num_actual_groups=np.asarray(A).shape[0], **kw)  # :401
     else:
-        dA = tgmm(dout, x, group_sizes, out_dtype=out_dtype, acc=acc)
+        dA = tgmm(dout, x, group_sizes, num_actual_groups=np.asarray(A).shape[0], **kw)
     return dx, dA, None
 
 

@@ -369,3 +369,71 @@ def test_short_group_row_tiles(k, split_k, trans_rhs):
         assert not torch.any(y[target_m:])
         assert prev is None or torch.equal(prev, y)
         prev = y
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# a slice of the groups (group_offset of jax.lax.ragged_dot; an expert-parallel rank's share of the weights)
+# ---------------------------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("o,gl", [(0, 9), (3, 4), (5, 4), (8, 1), (1, 1)], ids=lambda v: str(v))
+def test_group_offset_forward_and_vjp(o, gl, dtype):
+    """gmm / tgmm / the VJP with A holding groups [o, o + gl) of 9: against the oracle (pinned on the CPU as the product
+    with the other groups' weights zero); rows of the other groups and the tail exactly zero; shards add up to the
+    whole."""
+    m, k, n, G = 1500, 136, 264, 9
+    lhs, rhs, dout, _, _ = util.make_case(17, m, k, n, G, 1.0, True, scale_rhs=True)
+    gs = np.array([300, 0, 17, 450, 1, 212, 0, 260, 90], np.int32)  # 1330 of 1500 rows
+    target_m = int(gs.sum())
+    if dtype == "bf16":
+        dev, kw, eps = util.bf16_dev, {}, util.BF16_EPS
+    else:
+        rng = np.random.default_rng(3)
+        lhs, rhs, dout = (a + rng.normal(size=a.shape).astype(np.float32) * 1e-3 for a in (lhs, rhs, dout))
+        dev = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
+        kw, eps = dict(out_dtype="float32", acc=np.float64), 5e-4
+    gs_t = torch.from_numpy(gs)
+    off = np.concatenate([[0], np.cumsum(gs)])
+    inside = np.zeros(m, bool)
+    inside[off[o]:off[o + gl]] = True
+    for trans_rhs in (False, True):
+        print(f"group_offset o={o} gl={gl} {dtype} trans_rhs={trans_rhs}", flush=True)
+        A_np = rhs[o:o + gl]
+        A_in = np.ascontiguousarray(np.swapaxes(A_np, 1, 2)) if trans_rhs else A_np
+        x_t, A_t = dev(lhs).requires_grad_(True), dev(A_in).requires_grad_(True)
+        y = rd.gmm(x_t, A_t, gs_t, trans_rhs=trans_rhs, group_offset=o)
+        dx, dA = torch.autograd.grad(y, (x_t, A_t), dev(dout))
+        y_ref = oracle.gmm(lhs, A_in, gs, trans_rhs=trans_rhs, group_offset=o, **kw)
+        dx_ref, dA_ref, _ = oracle.gmm_vjp(lhs, A_in, gs, dout, trans_rhs=trans_rhs, group_offset=o, **kw)
+        for name, got, ref in (("y", y, y_ref), ("dx", dx, dx_ref)):
+            got = util.to_np(got)
+            assert float(np.max(oracle.err_fn(got, ref, mask=inside))) < eps, name
+            assert not np.any(got[~inside]), f"{name}: rows of groups outside the slice (and the tail) must be zero"
+        dA = util.to_np(dA)
+        assert dA.shape == dA_ref.shape == A_in.shape
+        assert float(np.max(oracle.err_fn(dA, dA_ref, axis=(-1, -2), mask=gs[o:o + gl] != 0))) < eps
+        assert not np.any(dA[gs[o:o + gl] == 0])
+    # tgmm's public keywords
+    out = rd.tgmm(dev(lhs), dev(dout), gs_t, group_offset=o, num_actual_groups=gl)
+    ref = oracle.tgmm(lhs, dout, gs, group_offset=o, num_actual_groups=gl, **kw)
+    assert float(np.max(oracle.err_fn(util.to_np(out), ref, axis=(-1, -2), mask=gs[o:o + gl] != 0))) < eps
+
+
+def test_group_offset_shards_add_up_and_bad_slices_are_refused():
+    m, k, n, G = 1024, 256, 512, 8
+    lhs, rhs, _, gs, target_m = util.make_case(23, m, k, n, G, 0.9, True, scale_rhs=True)
+    x, A, gs_t = util.bf16_dev(lhs), util.bf16_dev(rhs), torch.from_numpy(gs)
+    whole = rd.gmm(x, A, gs_t)
+    parts = [rd.gmm(x, A[o:o + 2].contiguous(), gs_t, group_offset=o) for o in (0, 2, 4, 6)]
+    assert torch.equal(sum(p.float() for p in parts), whole.float())  # disjoint row sets: exact
+    y = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    ws = torch.empty(_capi.lib.rd_gmm_workspace_bytes(m, G, None), dtype=torch.uint8, device="cuda")
+    for o, gl in ((7, 2), (-1, 2), (0, 0), (8, 1)):
+        rc = _capi.lib.rd_gmm_sharded(_stream(), x.data_ptr(), A.data_ptr(), gs_t.cuda().data_ptr(), y.data_ptr(), m, k, n,
+                                      G, o, gl, 0, _capi.RD_DTYPE_BF16, None, ws.data_ptr(), ws.numel())
+        assert rc == _capi.RD_ERR_INVALID_ARGUMENT, (o, gl, rc)
+    plan = _capi.Plan(-1, 0, 64)  # a streaming kernel on a slice: refused
+    rc = _capi.lib.rd_gmm_sharded(_stream(), x.data_ptr(), A.data_ptr(), gs_t.cuda().data_ptr(), y.data_ptr(), m, k, n, G, 2, 2,
+                                  0, _capi.RD_DTYPE_BF16, ctypes.byref(plan), ws.data_ptr(), ws.numel())
+    assert rc == _capi.RD_ERR_UNSUPPORTED
+    torch.cuda.synchronize()

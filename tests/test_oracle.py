@@ -232,6 +232,29 @@ def test_tgmm_vjp_adjoint_identities_and_finite_differences():
     np.testing.assert_allclose(dy[23:27], x[23:27] @ dout[3], rtol=1e-12)
 
 
+def test_group_offset_is_the_product_with_the_other_groups_weights_zero():
+    """group_offset (A holds a slice of the groups) reduces to the pinned definition: the same product with zero
+    weights for the groups outside the slice; tgmm's slices are rows [o, o + gl) of the full result; the VJP wiring
+    satisfies the adjoint identities."""
+    rng = np.random.default_rng(8)
+    m, k, n, G = 40, 6, 5, 7
+    gs = [5, 0, 9, 3, 8, 0, 10]  # 35 of 40 rows
+    x, A, dy = rng.normal(size=(m, k)), rng.normal(size=(G, k, n)), rng.normal(size=(m, n))
+    f64 = dict(out_dtype="float32", acc=np.float64)
+    for o, gl in ((0, 7), (2, 3), (4, 3), (6, 1), (1, 1)):
+        A0 = np.zeros_like(A)
+        A0[o:o + gl] = A[o:o + gl]
+        np.testing.assert_array_equal(oracle.gmm(x, A[o:o + gl], gs, group_offset=o, **f64), oracle.gmm(x, A0, gs, **f64))
+        At = np.swapaxes(A, 1, 2).copy()
+        np.testing.assert_array_equal(oracle.gmm(x, At[o:o + gl], gs, trans_rhs=True, group_offset=o, **f64), oracle.gmm(x, A0, gs, **f64))
+        np.testing.assert_array_equal(oracle.tgmm(x, dy, gs, group_offset=o, num_actual_groups=gl, **f64), oracle.tgmm(x, dy, gs, **f64)[o:o + gl])
+        dx, dA, _ = oracle.gmm_vjp(x, A[o:o + gl], gs, dy, group_offset=o, **f64)
+        s = np.sum(dy * oracle.gmm(x, A[o:o + gl], gs, group_offset=o, **f64))
+        np.testing.assert_allclose(np.sum(dx * x), s, rtol=1e-10)
+        np.testing.assert_allclose(np.sum(dA * A[o:o + gl]), s, rtol=1e-10)
+        assert dA.shape == (gl, k, n)
+
+
 # ---- the loop-nest restatement against the definition, on the reference's own grid ----------------------------------
 
 GRID = util.reference_grid(36, seed=1)
