@@ -156,7 +156,13 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
   SplitK sk;
   int k0 = 0, klen = p.k;
   if ((int)blockIdx.x < p.main_grid) {
-    const int per_block = p.group_m * p.group_n;
+    // With only a few rounds of tiles, blocks of the full size would leave some XCDs without work (180 tiles in blocks
+    // of 32 occupy 6 of the 8): the blocks shrink so that every round deals one to each XCD.
+    int per_block = p.group_m * p.group_n;
+    if (live < 4 * p.num_cus) {
+      const int rounds = (live + p.num_cus - 1) / p.num_cus;
+      per_block = imax(1, imin(per_block, (live + 8 * rounds - 1) / (8 * rounds)));
+    }
     const int pos = blockIdx.x >> 3;
     const int block = (pos / per_block) * 8 + (blockIdx.x & 7);
     t = block * per_block + pos % per_block;
@@ -297,10 +303,10 @@ int launch_gmm(hipStream_t s, const GmmArgs& a) {
   auto kern = gmm_kernel<C, TRANS_RHS>;
   const int attr_rc = allow_big_lds(reinterpret_cast<const void*>(kern), C::LDS_BYTES);
   if (attr_rc != hipSuccess) return attr_rc;
+  // positions per XCD: enough for any block size the kernel may shrink to (at most group_m x group_n)
   const int per_block = a.group_m * a.group_n;
-  const int blocks = (a.U * a.n_tiles + per_block - 1) / per_block;
   GmmArgs args = a;
-  args.main_grid = 8 * ((blocks + 7) / 8) * per_block;
+  args.main_grid = 8 * ((a.U * a.n_tiles + 7) / 8 + 2 * per_block);
   if (!C::SPLITK) args.split_slots = 0;
   const int grid = args.main_grid + args.split_slots;
   if (args.main_grid <= 0) return hipSuccess;
