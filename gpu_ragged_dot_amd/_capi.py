@@ -20,6 +20,7 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libragged_dot_hip.so")
 RD_DTYPE_BF16 = 0
 RD_DTYPE_F32 = 1
 RD_DTYPE_F32_BF16 = 2  # float32 arrays rounded to bfloat16 for the bf16 matrix cores (compute_dtype=bfloat16)
+RD_DTYPE_F8E4M3_BF16 = 3  # float8 e4m3fn operands widened to bfloat16 for the bf16 matrix cores, bfloat16 out
 
 RD_OK = 0
 RD_ERR_INVALID_ARGUMENT = -1

@@ -8,6 +8,7 @@ namespace rd {
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef short s16x8_t __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -23,6 +24,22 @@ __device__ __forceinline__ bf16_bits f32_to_bf16(float f) {
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+
+typedef uint8_t fp8_bits;  // storage type of an OCP float8 e4m3fn element in HBM
+
+// float8 e4m3fn (1 sign, 4 exponent bits of bias 7, 3 mantissa bits; no infinities, S.1111.111 is NaN) -> bf16.  Every
+// e4m3 value is a bf16 value, so this is exact: the hardware widens to fp32 (gfx950's float8 is this format) and the
+// upper half of the fp32 word is the bf16.
+// The two float8 bytes of the lower (HI = false) or upper half of w, as a pair of bf16.
+template <bool HI>
+__device__ __forceinline__ uint32_t fp8e4m3x2_to_bf16x2(uint32_t w) {
+  const f32x2_t f = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, HI);
+  // bytes 2-3 of each fp32 word: [f[1].b3 f[1].b2 f[0].b3 f[0].b2]
+  return __builtin_amdgcn_perm(__float_as_uint(f[1]), __float_as_uint(f[0]), 0x07060302u);
+}
+__device__ __forceinline__ uint32_t fp8e4m3_to_bf16(uint32_t b) {
+  return fp8e4m3x2_to_bf16x2<false>(b & 0xff) & 0xffff;
 }
 
 __device__ __forceinline__ float bf16_to_f32(bf16_bits b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }

@@ -13,6 +13,7 @@
 // Raggedness: a tile never spans two groups.  Rows/columns of the tile past its limit are fetched from a clamped
 // (always valid) address and simply not stored; only the contraction remainder is zero-filled.
 #pragma once
+#include <type_traits>
 #include "rd_common.h"
 
 namespace rd {
@@ -20,11 +21,13 @@ namespace rd {
 // Src: element type of the operands and the output in HBM.  bf16_bits: bf16 in, bf16 out.  float: float32 arrays whose
 // elements are rounded to bf16 (nearest even) on their way into LDS, multiplied on the bf16 matrix cores with fp32
 // accumulation and stored as float32 - the reference's compute_dtype = bfloat16 on float32 arrays
-// (gpu_ragged_dot.py:116-119, 145, 149).
+// (gpu_ragged_dot.py:116-119, 145, 149).  fp8_bits: float8 e4m3fn operands, widened (exactly) to bf16 on their way into
+// LDS, bf16 matrix cores with fp32 accumulation, bf16 out.
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, bool A_KMAJOR_, bool B_KMAJOR_, bool VEC_,
           typename Src = bf16_bits>
 struct TileCfg {
   typedef Src Elem;
+  typedef typename std::conditional<sizeof(Src) == 1, bf16_bits, Src>::type Out;  // element type of the output
   static constexpr bool F32 = false;
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
   static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = VEC_, DLDS = false, PINGPONG = false, MIXED = false,
@@ -66,13 +69,20 @@ struct OperandStager {
   static __device__ __forceinline__ u32x4_t chunk8(const Src* p) {
     if constexpr (sizeof(Src) == 2) {
       return *reinterpret_cast<const u32x4_t*>(p);
+    } else if constexpr (sizeof(Src) == 1) {
+      const u32x2_t raw = *reinterpret_cast<const u32x2_t*>(p);  // 8 bytes: p is 8-byte aligned
+      const u32x4_t r = {fp8e4m3x2_to_bf16x2<false>(raw[0]), fp8e4m3x2_to_bf16x2<true>(raw[0]),
+                         fp8e4m3x2_to_bf16x2<false>(raw[1]), fp8e4m3x2_to_bf16x2<true>(raw[1])};
+      return r;
     } else {
       const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(p), hi = *reinterpret_cast<const f32x4_t*>(p + 4);
       return u32x4_t{pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]), pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3])};
     }
   }
   static __device__ __forceinline__ bf16_bits elem(const Src* p) {
-    if constexpr (sizeof(Src) == 2) return *p; else return f32_to_bf16(*p);
+    if constexpr (sizeof(Src) == 2) return *p;
+    else if constexpr (sizeof(Src) == 1) return (bf16_bits)fp8e4m3_to_bf16(*p);
+    else return f32_to_bf16(*p);
   }
 
   __device__ __forceinline__ void init(const Src* p, int ld_, int lim_, int klen_, int tid) {
@@ -152,7 +162,7 @@ __device__ __forceinline__ bf16x8_t read_fragment(const bf16_bits* lds, int idx0
 template <class C>
 __device__ __forceinline__ void gemm_tile(const typename C::Elem* __restrict__ Ap, int lda, int a_lim,
                                           const typename C::Elem* __restrict__ Bp, int ldb, int b_lim, int klen,
-                                          typename C::Elem* __restrict__ Op, int ldo, bf16_bits* smem) {
+                                          typename C::Out* __restrict__ Op, int ldo, bf16_bits* smem) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;
 
@@ -224,7 +234,7 @@ __device__ __forceinline__ void gemm_tile(const typename C::Elem* __restrict__ A
       for (int v = 0; v < 16; ++v) {
         const int row = wm * C::WM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
         if (row < a_lim && col < b_lim) {
-          if constexpr (sizeof(typename C::Elem) == 2) Op[(size_t)row * ldo + col] = f32_to_bf16(acc[i][j][v]);
+          if constexpr (sizeof(typename C::Out) == 2) Op[(size_t)row * ldo + col] = f32_to_bf16(acc[i][j][v]);
           else Op[(size_t)row * ldo + col] = acc[i][j][v];
         }
       }

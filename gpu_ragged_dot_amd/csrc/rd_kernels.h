@@ -56,9 +56,15 @@ struct IsW4 { static constexpr bool value = false; };
 template <class C>
 struct IsW4<C, decltype((void)C::W4)> { static constexpr bool value = true; };
 
+// Element type of a configuration's output: its Out when it names one (float8 operands give bf16), else that of its operands.
+template <class C, class = void>
+struct OutOf { typedef typename C::Elem type; };
+template <class C>
+struct OutOf<C, decltype((void)sizeof(typename C::Out))> { typedef typename C::Out type; };
+
 template <class C>
 __device__ __forceinline__ void run_tile(const typename C::Elem* Ap, int lda, int a_lim, const typename C::Elem* Bp,
-                                         int ldb, int b_lim, int klen, typename C::Elem* Op, int ldo,
+                                         int ldb, int b_lim, int klen, typename OutOf<C>::type* Op, int ldo,
                                          typename C::Elem* smem, const SplitK& sk = SplitK()) {
   if constexpr (C::F32) gemm_tile_f32<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
   else if constexpr (IsW4<C>::value) gemm_tile_w4<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
@@ -139,7 +145,8 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
   E* smem = reinterpret_cast<E*>(smem_raw);
   const E* px = static_cast<const E*>(p.x);
   const E* pA = static_cast<const E*>(p.A);
-  E* py = static_cast<E*>(p.y);
+  typedef typename OutOf<C>::type O;
+  O* py = static_cast<O*>(p.y);
   // Tile walk.  The scheduling-map kernel has cut every group's row tiles into bands of at most group_m row tiles
   // (tile2band); the walk visits band after band and, inside a band, column after column (all the band's row tiles of
   // one column tile, then the next column).  Position t of the walk therefore lies in the band of row tile t / n_tiles.
@@ -203,11 +210,11 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
     int rows = imin(C::BM, uniform(p.group_sizes[gi]) - it * C::BM);
     rows = imin(rows, p.m - row0);  // group_sizes summing past m: never touch rows >= m
     if (rows <= 0 || row0 < 0) return;
-    E* Op = py + (size_t)row0 * p.n + col0;
+    O* Op = py + (size_t)row0 * p.n + col0;
     const int gl = gi - p.g_first;  // index of the group's weights in A
     if (gl < 0 || gl >= p.g_local) {
       // a group whose weights live elsewhere (A is a slice of the groups): its rows of y are zero
-      if (sk.part == 0) zero_tile<C::NT, C::VEC, E>(Op, p.n, rows, cols);
+      if (sk.part == 0) zero_tile<C::NT, C::VEC, O>(Op, p.n, rows, cols);
       return;
     }
     const E* Ap = px + (size_t)row0 * p.k + k0;
@@ -237,7 +244,7 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
     const long long r0 = s + (long long)(mi - total) * C::BM;
     if (r0 >= p.m) return;
     const int rows = imin(C::BM, p.m - (int)r0);
-    zero_tile<C::NT, C::VEC, E>(py + (size_t)r0 * p.n + col0, p.n, rows, cols);
+    zero_tile<C::NT, C::VEC, O>(py + (size_t)r0 * p.n + col0, p.n, rows, cols);
   }
 }
 
@@ -261,13 +268,14 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void tgmm_kernel(TgmmArgs p
 
   const int kk0 = ri * C::BM, col0 = cj * C::BN;
   const int krows = imin(C::BM, p.k - kk0), cols = imin(C::BN, p.n - col0);
-  E* Op = static_cast<E*>(p.dA) + (size_t)gi * p.k * p.n + (size_t)kk0 * p.n + col0;
+  typedef typename OutOf<C>::type O;
+  O* Op = static_cast<O*>(p.dA) + (size_t)gi * p.k * p.n + (size_t)kk0 * p.n + col0;
 
   const int row0 = uniform(p.group_offsets[gi + p.g_first]);
   int rows = uniform(p.group_sizes[gi + p.g_first]);
   rows = imin(rows, p.m - row0);
   if (rows <= 0 || row0 < 0) {  // empty group: its slice of dA is zero
-    zero_tile<C::NT, C::VEC, E>(Op, p.n, krows, cols);
+    zero_tile<C::NT, C::VEC, O>(Op, p.n, krows, cols);
     return;
   }
   const E* Ap = static_cast<const E*>(p.x) + (size_t)row0 * p.k + kk0;

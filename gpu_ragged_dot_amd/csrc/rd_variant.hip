@@ -1,6 +1,6 @@
 // One compiled tile shape.  Built once per entry of the variant list in the Makefile, with
 //   -DRD_BM= -DRD_BN= -DRD_BK= -DRD_WAVES_M= -DRD_WAVES_N= -DRD_VEC= -DRD_NAME= [-DRD_DLDS=1|2|3 -DRD_STAGES= -DRD_PINGPONG=1
-//   -DRD_F32=1|2]
+//   -DRD_F32=1|2|3]
 // and exports a getter rd_variant_<name>() for its TileVariant record that the C-ABI file collects.
 #include "rd_kernels.h"
 
@@ -24,7 +24,12 @@
 #endif
 
 namespace rd {
-#if RD_F32 == 2
+#if RD_F32 == 3
+// float8 e4m3fn arrays, widened to bf16 on the way into LDS, bf16 matrix cores, bf16 out
+typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, /*A K-major*/ true, /*B K-major*/ false, RD_VEC != 0, fp8_bits> CfgNN;
+typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, true, true, RD_VEC != 0, fp8_bits> CfgNT;
+typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, false, false, RD_VEC != 0, fp8_bits> CfgTN;
+#elif RD_F32 == 2
 // float32 arrays, rounded to bf16 on the way into LDS, bf16 matrix cores, float32 out (compute_dtype = bfloat16)
 typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, /*A K-major*/ true, /*B K-major*/ false, RD_VEC != 0, float> CfgNN;
 typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, true, true, RD_VEC != 0, float> CfgNT;

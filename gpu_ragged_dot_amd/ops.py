@@ -17,16 +17,27 @@ from .planner import CHUNK_M, DEFAULT_BLOCK_K, DEFAULT_BLOCK_M, DEFAULT_BLOCK_N
 
 __all__ = ["gmm", "tgmm", "ragged_dot", "trans_ragged_dot", "ragged_dot_vjp", "make_group_metadata"]
 
-_DTYPES = {torch.bfloat16: _capi.RD_DTYPE_BF16, torch.float32: _capi.RD_DTYPE_F32}
+_DTYPES = {torch.bfloat16: _capi.RD_DTYPE_BF16, torch.float32: _capi.RD_DTYPE_F32,
+           torch.float8_e4m3fn: _capi.RD_DTYPE_F8E4M3_BF16}
+
+
+def _out_dtype(t: torch.Tensor) -> torch.dtype:
+    """The output has the operands' element type (gpu_ragged_dot.py:210,324); float8 operands, which the reference does
+    not have, give bfloat16 (jax.lax.ragged_dot with preferred_element_type=bfloat16)."""
+    return torch.bfloat16 if t.dtype == torch.float8_e4m3fn else t.dtype
 
 
 def _dtype_code(t: torch.Tensor, compute_dtype, acc_dtype) -> int:
     """Element-type code for the C ABI from the storage dtype and the reference's ``compute_dtype``
     (gpu_ragged_dot.py:116-119, 145: operands are cast to compute_dtype before the dot; None = the storage dtype)."""
     if t.dtype not in _DTYPES:
-        raise TypeError(f"unsupported dtype {t.dtype}; operands are bfloat16 or float32")
+        raise TypeError(f"unsupported dtype {t.dtype}; operands are bfloat16, float32 or float8_e4m3fn")
     if acc_dtype not in (None, torch.float32):
         raise NotImplementedError("accumulation is always float32 on the matrix cores")
+    if t.dtype == torch.float8_e4m3fn:
+        if compute_dtype not in (None, torch.bfloat16, torch.float32, torch.float8_e4m3fn):
+            raise NotImplementedError(f"no kernel for compute_dtype={compute_dtype} on float8 operands")
+        return _capi.RD_DTYPE_F8E4M3_BF16  # float8 products are exact in every one of these types; accumulation is fp32
     if compute_dtype is None or compute_dtype == t.dtype:
         return _DTYPES[t.dtype]
     if t.dtype == torch.float32 and compute_dtype == torch.bfloat16:
@@ -110,7 +121,7 @@ def _gmm_fwd(x, A, group_sizes, block_m, block_k, block_n, trans_rhs, interpret,
         raise TypeError(f"x is {x.dtype} but A is {A.dtype}")
     x, A = x.contiguous(), A.contiguous()
     gs = _group_sizes_i32(group_sizes, dev)
-    y = torch.empty((m, n), dtype=x.dtype, device=dev)  # :210
+    y = torch.empty((m, n), dtype=_out_dtype(x), device=dev)  # :210
     if plan is None:
         plan = planner.select_plan(_capi.OP_GMM_TRANS if trans_rhs else _capi.OP_GMM, m, k, n, g, block_m, block_k, block_n,
                                    dtype=code, aligned=_aligned16(x, A, y))
@@ -148,7 +159,7 @@ def _tgmm_fwd(x, y, group_sizes, block_m, block_k, block_n, interpret, compute_d
     g_first = _group_offset(group_offset)
     g_local = g - g_first if num_actual_groups is None else int(num_actual_groups)
     assert 0 <= g_first and g_local >= 1 and g_first + g_local <= g, f"groups [{g_first}, {g_first}+{g_local}) are not within {g}"
-    out = torch.empty((g_local, k, n), dtype=x.dtype, device=dev)  # :324
+    out = torch.empty((g_local, k, n), dtype=_out_dtype(x), device=dev)  # :324
     if plan is None:
         plan = planner.select_plan(_capi.OP_TGMM, m, k, n, g, block_m, block_k, block_n, dtype=code,
                                    aligned=_aligned16(x, y, out))
@@ -241,6 +252,8 @@ def gmm(
     if group_offset is not None:
         hp["group_offset"] = _group_offset(group_offset)
     if torch.is_grad_enabled() and (x.requires_grad or A.requires_grad):
+        if x.dtype == torch.float8_e4m3fn:
+            raise NotImplementedError("float8 operands are forward only: their cotangents are bfloat16, differentiate a bfloat16 copy")
         gs = _group_sizes_i32(group_sizes, x.device)
         return _GmmFn.apply(x, A, gs, hp)
     return _gmm_fwd(x, A, group_sizes, **hp)

@@ -9,7 +9,8 @@
  *    workspace; the library never allocates or frees device memory and never synchronises;
  *  - `stream` is a hipStream_t passed as void* (NULL = the default stream);
  *  - matrices are dense row-major; element type is selected by `dtype` (RD_DTYPE_*), output type = input type
- *    (gpu_ragged_dot.py:210,324), accumulation is always fp32 (acc_dtype, gpu_ragged_dot.py:119,251);
+ *    (gpu_ragged_dot.py:210,324; the float8 type, which the reference does not have, gives bfloat16), accumulation is
+ *    always fp32 (acc_dtype, gpu_ragged_dot.py:119,251);
  *  - return value 0 = success; negative = RD_ERR_*; the text of the last error of the calling thread is
  *    available from rd_last_error().  Nothing here aborts the process;
  *  - no host reads of device data: the launch grid is the static bound ceil(m / tile_m) + g of
@@ -27,12 +28,19 @@ extern "C" {
 
 #define RD_ABI_VERSION 2
 
-/* Element type of the operands and the output (always the same, gpu_ragged_dot.py:210,324) and what the matrix cores
- * multiply.  RD_DTYPE_F32_BF16 is compute_dtype = bfloat16 on float32 arrays (gpu_ragged_dot.py:116-119, 145, 149): the
+/* Element type of the operands and the output (the same, gpu_ragged_dot.py:210,324, but for float8) and what the matrix
+ * cores multiply.  RD_DTYPE_F32_BF16 is compute_dtype = bfloat16 on float32 arrays (gpu_ragged_dot.py:116-119, 145, 149): the
  * float32 elements are rounded to bfloat16 (nearest even) as they are loaded, multiplied on the bf16 matrix cores with
  * fp32 accumulation, and stored as float32.  (compute_dtype = float32 on bfloat16 arrays is RD_DTYPE_BF16 itself: a
- * product of two bfloat16 values is exact in fp32, and the accumulation is fp32 either way.) */
-enum rd_dtype { RD_DTYPE_BF16 = 0, RD_DTYPE_F32 = 1, RD_DTYPE_F32_BF16 = 2 };
+ * product of two bfloat16 values is exact in fp32, and the accumulation is fp32 either way.)
+ * RD_DTYPE_F8E4M3_BF16: both operands (x and A of rd_gmm, x and dy of rd_tgmm) are float8 e4m3fn bytes (the OCP format:
+ * bias 7, no infinities, 0x7f / 0xff are NaN), the output is bfloat16 - jax.lax.ragged_dot on float8 operands with
+ * preferred_element_type = bfloat16; the reference itself has no float8 path.  The bytes are widened to bfloat16 as
+ * they are loaded (exact: every e4m3 value is a bfloat16 value) and multiplied on the bf16 matrix cores with fp32
+ * accumulation, so the result is that of an exact-product fp32-accumulating float8 multiply; what float8 buys here is
+ * half the bytes read, not a higher matrix-core rate.  Tile kernels only (no streaming kernel for a few rows per
+ * group, no K-split). */
+enum rd_dtype { RD_DTYPE_BF16 = 0, RD_DTYPE_F32 = 1, RD_DTYPE_F32_BF16 = 2, RD_DTYPE_F8E4M3_BF16 = 3 };
 
 #define RD_DECODE_ROWS (-1) /* rd_plan.decode_nb: the streaming kernel that cuts each expert's weights into whole-row slices */
 

@@ -63,6 +63,32 @@ def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
     return (np.ascontiguousarray(b, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
 
 
+def float8_e4m3fn_to_f32(b: np.ndarray) -> np.ndarray:
+    """float8 e4m3fn bit patterns (uint8) -> float32 values, by the format's definition (OCP 8-bit floating point
+    specification, E4M3: 1 sign, 4 exponent bits of bias 7, 3 mantissa bits; exponent 0 holds zero and the subnormals
+    mantissa x 2^-9; there are no infinities, S.1111.111 is NaN; largest finite value 448).  Not in the reference, which
+    has no float8 path: this is the element type of jax.lax.ragged_dot's float8 variants."""
+    b = np.ascontiguousarray(b, dtype=np.uint8).astype(np.int64)
+    sign = np.where(b & 0x80, -1.0, 1.0)
+    e, mant = (b >> 3) & 0xF, b & 0x7
+    mag = np.where(e == 0, mant * 2.0 ** -9, (1.0 + mant / 8.0) * np.exp2((e - 7).astype(np.float64)))
+    return np.where((b & 0x7F) == 0x7F, np.nan, sign * mag).astype(np.float32)
+
+
+def f32_to_float8_e4m3fn(a: np.ndarray) -> np.ndarray:
+    """float -> nearest float8 e4m3fn bit pattern (uint8), ties to the even code, magnitudes beyond 448 saturating to
+    448 and NaN to 0x7f: a search over the 127 non-negative finite codes, for making test inputs."""
+    a = np.asarray(a, dtype=np.float64)
+    table = float8_e4m3fn_to_f32(np.arange(127, dtype=np.uint8)).astype(np.float64)  # increasing
+    mag = np.minimum(np.abs(a), 448.0)
+    hi = np.clip(np.searchsorted(table, mag), 1, 126)
+    lo = hi - 1
+    d_lo, d_hi = mag - table[lo], table[hi] - mag
+    code = np.where(d_lo < d_hi, lo, np.where(d_hi < d_lo, hi, np.where(lo % 2 == 0, lo, hi)))
+    code = np.where(np.isnan(a), 0x7F, code)
+    return (code | np.where(np.signbit(a), 0x80, 0)).astype(np.uint8)
+
+
 def round_to(a: np.ndarray, dtype: str) -> np.ndarray:
     """Round a float array to ``dtype`` ('bfloat16' | 'float32') and return it as float32 values."""
     if dtype == "bfloat16":

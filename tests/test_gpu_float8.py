@@ -1,0 +1,148 @@
+"""GPU parity for float8 e4m3fn operands (jax.lax.ragged_dot's float8 variant; the reference has no float8 path): the
+HIP kernels widen the bytes to bf16 on their way into LDS, multiply on the bf16 matrix cores with fp32 accumulation and
+store bf16.  Everything goes through the C ABI (ctypes).  The oracle decodes the bytes by the format's definition and
+computes in float64; since products of two e4m3 values are exact in fp32, what is left is the fp32 accumulation order
+and the bf16 rounding of the result: the bf16 tolerances of the other parity tests apply unchanged."""
+
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import gpu_ragged_dot_amd as rd
+from gpu_ragged_dot_amd import _capi, ops
+from oracle import ragged_dot_oracle as oracle
+from tests import util
+
+pytestmark = pytest.mark.gpu
+
+HP = dict(block_m=64, block_k=64, block_n=64, interpret=False, compute_dtype=None, acc_dtype=torch.float32, chunk_m=512)
+TGMM_EPS = 2e-2  # as the bf16 tgmm tests: rel-Frobenius per group slice
+
+
+def _f8_dev(codes: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(np.ascontiguousarray(codes)).cuda().view(torch.float8_e4m3fn)
+
+
+def _case(seed, m, k, n, g, fill=0.9):
+    rng = np.random.default_rng(seed)
+    target_m = int(m * fill)
+    gs = oracle.generate_group_sizes(seed, g, target_m)
+    x8 = oracle.f32_to_float8_e4m3fn(rng.normal(size=(m, k)))
+    A8 = oracle.f32_to_float8_e4m3fn(rng.normal(size=(g, k, n)) / np.sqrt(k))  # many subnormals among these
+    d8 = oracle.f32_to_float8_e4m3fn(rng.normal(size=(m, n)))
+    return x8, A8, d8, gs, target_m
+
+
+def _f8_variants():
+    return [v for v in _capi.variants() if v.dtype == _capi.RD_DTYPE_F8E4M3_BF16]
+
+
+def test_every_code_passes_through_exactly():
+    """x holds every finite code, A is a stack of identity matrices (1.0 = 0x38): y is x, exactly, as bf16."""
+    k = 256
+    codes = np.arange(256, dtype=np.uint8)
+    finite = np.where((codes & 0x7F) == 0x7F, 0, codes)
+    rng = np.random.default_rng(3)
+    x8 = np.stack([np.roll(finite, s) for s in range(0, 96)] + [rng.permutation(finite) for _ in range(96)])  # [192, 256]
+    eye = np.zeros((3, k, k), np.uint8)
+    eye[:, np.arange(k), np.arange(k)] = 0x38
+    gs = np.array([100, 0, 92], np.int32)
+    want = oracle.float8_e4m3fn_to_f32(x8)
+    for trans_rhs in (False, True):
+        y = rd.gmm(_f8_dev(x8), _f8_dev(eye), torch.from_numpy(gs), trans_rhs=trans_rhs)
+        assert y.dtype == torch.bfloat16
+        assert np.array_equal(util.to_np(y), want), f"trans_rhs={trans_rhs}"
+    # a NaN code poisons exactly its own row
+    x8[5, 17] = 0x7F
+    x8[150, 0] = 0xFF
+    y = util.to_np(rd.gmm(_f8_dev(x8), _f8_dev(eye), torch.from_numpy(gs)))
+    bad = np.isnan(y).any(axis=1)
+    assert bad[5] and bad[150] and bad.sum() == 2
+    assert np.isnan(y[5, 17]) and np.isnan(y[150, 0])
+
+
+SHAPES = [(512, 256, 384, 4), (1030, 264, 392, 5), (515, 99, 131, 3), (300, 64, 64, 7), (2048, 512, 1024, 16), (64, 1024, 256, 32)]
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "m%d_k%d_n%d_g%d" % s)
+def test_float8_products_against_the_oracle(shape):
+    """gmm (both layouts of A) and tgmm on ragged shapes with a zero tail and empty groups, default plan."""
+    m, k, n, g = shape
+    print("float8", shape, flush=True)
+    x8, A8, d8, gs, target_m = _case(m + g, m, k, n, g)
+    xf, Af, df = (oracle.float8_e4m3fn_to_f32(a) for a in (x8, A8, d8))
+    gs_t = torch.from_numpy(gs)
+    y_ref = oracle.gmm(xf, Af, gs)
+    y = rd.gmm(_f8_dev(x8), _f8_dev(A8), gs_t)
+    assert y.dtype == torch.bfloat16 and tuple(y.shape) == (m, n)
+    util.assert_close_rows(util.to_np(y), y_ref, target_m, util.BF16_EPS, "gmm")
+    assert not np.any(util.to_np(y)[target_m:])
+    At8 = np.ascontiguousarray(np.swapaxes(A8, 1, 2))
+    yt = rd.gmm(_f8_dev(x8), _f8_dev(At8), gs_t, trans_rhs=True)
+    util.assert_close_rows(util.to_np(yt), y_ref, target_m, util.BF16_EPS, "gmm trans_rhs")
+    dA_ref = oracle.tgmm(xf, df, gs)
+    dA = rd.tgmm(_f8_dev(x8), _f8_dev(d8), gs_t)
+    assert dA.dtype == torch.bfloat16 and tuple(dA.shape) == (g, k, n)
+    util.assert_close_groups(util.to_np(dA), dA_ref, gs != 0, TGMM_EPS, "tgmm")
+    assert not np.any(util.to_np(dA)[gs == 0])
+
+
+@pytest.mark.parametrize("shape", [(1030, 264, 392, 5), (515, 99, 131, 3)], ids=lambda s: "m%d_k%d_n%d_g%d" % s)
+def test_float8_every_tile_shape(shape):
+    """Each tile shape compiled for float8 operands, forced through the plan (the 8-byte-chunk ones only where the
+    pitches allow), for gmm, gmm trans_rhs and tgmm; output NaN-poisoned first, rows below the output untouched."""
+    m, k, n, g = shape
+    x8, A8, d8, gs, target_m = _case(7 + m, m, k, n, g)
+    xf, Af, df = (oracle.float8_e4m3fn_to_f32(a) for a in (x8, A8, d8))
+    y_ref, dA_ref = oracle.gmm(xf, Af, gs), oracle.tgmm(xf, df, gs)
+    x, A, d = _f8_dev(x8), _f8_dev(A8), _f8_dev(d8)
+    At = _f8_dev(np.ascontiguousarray(np.swapaxes(A8, 1, 2)))
+    gs_d = torch.from_numpy(gs).cuda()
+    variants = _f8_variants()
+    assert len(variants) >= 2 and any(not v.vec for v in variants)
+    ran = 0
+    guard = 32
+    for v in variants:
+        if v.vec and (k % 8 or n % 8):
+            continue
+        print("float8 tile", v.name.decode(), shape, flush=True)
+        plan = _capi.Plan(v.id)
+        ws = torch.empty(max(_capi.lib.rd_gmm_workspace_bytes(m, g, ctypes.byref(plan)), 256), dtype=torch.uint8, device="cuda")
+        for trans_rhs, rhs in ((0, A), (1, At)):
+            y = torch.full((m + guard, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+            rc = _capi.lib.rd_gmm(torch.cuda.current_stream().cuda_stream, x.data_ptr(), rhs.data_ptr(), gs_d.data_ptr(),
+                                  y.data_ptr(), m, k, n, g, trans_rhs, _capi.RD_DTYPE_F8E4M3_BF16, ctypes.byref(plan),
+                                  ws.data_ptr(), ws.numel())
+            torch.cuda.synchronize()
+            assert rc == 0, _capi.lib.rd_last_error()
+            got = util.to_np(y)
+            assert np.isnan(got[m:]).all() and not np.isnan(got[:m]).any()
+            util.assert_close_rows(got[:m], y_ref, target_m, util.BF16_EPS, f"gmm {v.name.decode()} trans_rhs={trans_rhs}")
+            assert not np.any(got[target_m:m])
+        dA = ops._tgmm_fwd(x, d, gs_d, **HP, plan=plan)
+        util.assert_close_groups(util.to_np(dA), dA_ref, gs != 0, TGMM_EPS, f"tgmm {v.name.decode()}")
+        assert not np.any(util.to_np(dA)[gs == 0])
+        ran += 1
+    assert ran >= 1
+
+
+def test_float8_is_forward_only_and_rejects_mixed_operands():
+    x8, A8, _, gs, _ = _case(1, 128, 64, 64, 2)
+    x, A = _f8_dev(x8), _f8_dev(A8)
+    gs_t = torch.from_numpy(gs)
+    with pytest.raises(TypeError):
+        rd.gmm(x, A.to(torch.bfloat16), gs_t)
+    with pytest.raises(NotImplementedError):
+        rd.gmm(x, A, gs_t, compute_dtype=torch.float16)
+    try:
+        xr = x.clone().requires_grad_(True)
+    except RuntimeError:
+        return  # this torch does not let a float8 tensor require a gradient at all
+    with pytest.raises(NotImplementedError):
+        rd.gmm(xr, A, gs_t)
+    # a bf16 variant forced on float8 operands is refused with a status code
+    bf16 = [v.id for v in _capi.variants() if v.dtype == _capi.RD_DTYPE_BF16][0]
+    with pytest.raises(_capi.RaggedDotError):
+        ops._gmm_fwd(x, A, gs_t, **HP, trans_rhs=False, plan=_capi.Plan(bf16))

@@ -304,3 +304,40 @@ def test_generate_group_sizes_sums():
         for g, t in ((8, 128), (16, 120), (16, 0), (8, 86)):
             gs = oracle.generate_group_sizes(seed, g, t)
             assert gs.dtype == np.int32 and gs.sum() == t and np.all(gs >= 0) and gs.size == g
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# float8 e4m3fn on the host
+# ---------------------------------------------------------------------------------------------------------------------
+
+def test_float8_decode_known_values_and_torch():
+    """Values fixed by the E4M3 definition (bias 7, subnormals mantissa x 2^-9, max 448, S.1111.111 NaN, no infinities),
+    then all 256 codes against torch's own CPU conversion - an independent implementation."""
+    torch = pytest.importorskip("torch")
+    dec = oracle.float8_e4m3fn_to_f32
+    known = {0x00: 0.0, 0x01: 2.0 ** -9, 0x07: 7 * 2.0 ** -9, 0x08: 2.0 ** -6, 0x0F: 1.875 * 2.0 ** -6, 0x38: 1.0, 0x3C: 1.5,
+             0x40: 2.0, 0x77: 1.875 * 2.0 ** 7, 0x78: 256.0, 0x7E: 448.0, 0xB8: -1.0, 0xFE: -448.0, 0x81: -(2.0 ** -9)}
+    for code, val in known.items():
+        assert float(dec(np.array([code], np.uint8))[0]) == val, hex(code)
+    assert np.signbit(dec(np.array([0x80], np.uint8))[0]) and dec(np.array([0x80], np.uint8))[0] == 0.0
+    assert np.isnan(dec(np.array([0x7F, 0xFF], np.uint8))).all()
+    codes = np.arange(256, dtype=np.uint8)
+    mine = dec(codes)
+    assert np.isfinite(mine).sum() == 254 and np.all(np.diff(mine[:127]) > 0)
+    theirs = torch.from_numpy(codes).view(torch.float8_e4m3fn).to(torch.float32).numpy()
+    assert np.array_equal(np.isnan(mine), np.isnan(theirs))
+    assert np.array_equal(mine[np.isfinite(mine)], theirs[np.isfinite(theirs)])
+    # every e4m3 value is a bf16 value: the kernels' widening is exact
+    assert np.array_equal(oracle.round_to(mine[np.isfinite(mine)], "bfloat16"), mine[np.isfinite(mine)])
+
+
+def test_float8_encode_round_trip_ties_and_saturation():
+    torch = pytest.importorskip("torch")
+    enc, dec = oracle.f32_to_float8_e4m3fn, oracle.float8_e4m3fn_to_f32
+    codes = np.arange(256, dtype=np.uint8)
+    finite = codes[(codes & 0x7F) != 0x7F]
+    assert np.array_equal(enc(dec(finite)), finite)
+    assert enc(np.array([1.0625]))[0] == 0x38 and enc(np.array([1.1875]))[0] == 0x3A  # ties go to the even code
+    assert enc(np.array([1e9]))[0] == 0x7E and enc(np.array([-1e9]))[0] == 0xFE and enc(np.array([np.nan]))[0] == 0x7F
+    x = (np.random.default_rng(0).normal(size=50000) * 4).astype(np.float32)
+    assert np.array_equal(enc(x), torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy())
