@@ -265,8 +265,10 @@ def bare_stream(copies, nbytes, torch):
 
 
 def dense_gemm_context(torch):
-    """hipBLASLt (torch.matmul) on one dense bf16 GEMM with the Mixtral forward's FLOPs, on N(0,1) data and on zeros:
-    what the vendor library reaches on this box, and how much the data (power) matters."""
+    """hipBLASLt (torch.matmul) on dense bf16 GEMMs with the FLOPs of one Mixtral product, on N(0,1) data and on zeros:
+    what the vendor library reaches on this box, and how much the data (power) matters.  Three operand layouts, those
+    of the three products: forward x[m,k].W[k,n]; dlhs dout[m,n].W[k,n]^T (both operands run along the contraction
+    index); drhs x[m,k]^T.dout[m,n]."""
     m, k, n = 16384, 4096, 14336
     gen = torch.Generator(device="cuda").manual_seed(7)
     out = {}
@@ -274,15 +276,23 @@ def dense_gemm_context(torch):
         if label == "normal":
             a = torch.randn((m, k), generator=gen, device="cuda").to(torch.bfloat16)
             b = (torch.randn((k, n), generator=gen, device="cuda") / k ** 0.5).to(torch.bfloat16)
+            d = torch.randn((m, n), generator=gen, device="cuda").to(torch.bfloat16)
         else:
             a = torch.zeros((m, k), dtype=torch.bfloat16, device="cuda")
             b = torch.zeros((k, n), dtype=torch.bfloat16, device="cuda")
+            d = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
         c = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
-        for _ in range(5):
-            torch.matmul(a, b, out=c)
-        ms = _event_ms(lambda: torch.matmul(a, b, out=c), 30, torch)
-        out[label] = {"ms": ms, "TFLOP/s": 2.0 * m * k * n / (ms * 1e-3) / 1e12}
-    return {"what": "torch.matmul bf16 [16384,4096]x[4096,14336] (the Mixtral forward's FLOPs as one dense GEMM)", **out}
+        ca = torch.empty((m, k), dtype=torch.bfloat16, device="cuda")
+        cb = torch.empty((k, n), dtype=torch.bfloat16, device="cuda")
+        layouts = (("", lambda: torch.matmul(a, b, out=c)), ("_dlhs_layout", lambda: torch.matmul(d, b.t(), out=ca)),
+                   ("_drhs_layout", lambda: torch.matmul(a.t(), d, out=cb)))
+        for suffix, fn in layouts:
+            for _ in range(5):
+                fn()
+            ms = _event_ms(fn, 30, torch)
+            out[label + suffix] = {"ms": ms, "TFLOP/s": 2.0 * m * k * n / (ms * 1e-3) / 1e12}
+    return {"what": "torch.matmul bf16, m16384 k4096 n14336: x.W (the Mixtral forward's FLOPs as one dense GEMM), "
+                    "dout.W^T (dlhs layout), x^T.dout (drhs layout)", **out}
 
 
 def bench_routing(args, torch):
