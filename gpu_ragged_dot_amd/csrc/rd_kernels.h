@@ -4,6 +4,7 @@
 #include "rd_gemm_dlds.h"
 #include "rd_gemm_f32.h"
 #include "rd_gemm_w4.h"
+#include "rd_gemm_w4r.h"
 #include "rd_gemm_pp.h"
 #include "rd_gemm_tile.h"
 #include "rd_sched.h"
@@ -55,6 +56,10 @@ template <class C, class = void>
 struct IsW4 { static constexpr bool value = false; };
 template <class C>
 struct IsW4<C, decltype((void)C::W4)> { static constexpr bool value = true; };
+template <class C, class = void>
+struct IsW4R { static constexpr bool value = false; };
+template <class C>
+struct IsW4R<C, decltype((void)C::W4R)> { static constexpr bool value = true; };
 
 // Element type of a configuration's output: its Out when it names one (float8 operands give bf16), else that of its operands.
 template <class C, class = void>
@@ -67,6 +72,7 @@ __device__ __forceinline__ void run_tile(const typename C::Elem* Ap, int lda, in
                                          int ldb, int b_lim, int klen, typename OutOf<C>::type* Op, int ldo,
                                          typename C::Elem* smem, const SplitK& sk = SplitK()) {
   if constexpr (C::F32) gemm_tile_f32<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
+  else if constexpr (IsW4R<C>::value) gemm_tile_w4r<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
   else if constexpr (IsW4<C>::value) gemm_tile_w4<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
   else if constexpr (C::MIXED) gemm_tile_pingpong_mixed<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
   else if constexpr (C::DLDS && C::PINGPONG) gemm_tile_pingpong<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);

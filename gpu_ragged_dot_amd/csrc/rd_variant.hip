@@ -40,7 +40,8 @@ typedef F32Cfg<RD_BM, RD_BN, true, true> CfgNT;
 typedef F32Cfg<RD_BM, RD_BN, false, false> CfgTN;
 #elif RD_DLDS == 3
 typedef W4Cfg<RD_BM, RD_BN, /*A K-major*/ true, /*B K-major*/ false, RD_STAGES> CfgNN;
-typedef W4Cfg<RD_BM, RD_BN, true, true, RD_STAGES> CfgNT;
+// both operands K-major: the 64-wide, register-staged form of the core (rd_gemm_w4r.h)
+typedef W4RCfg<RD_BM, RD_BN> CfgNT;
 typedef W4Cfg<RD_BM, RD_BN, false, false, RD_STAGES> CfgTN;
 #elif RD_DLDS == 2
 // one LDS ring per operand: one K-major operand in 64-wide slabs (3 slots) - the activations in the forward product,
