@@ -67,12 +67,19 @@ struct OutOf { typedef typename C::Elem type; };
 template <class C>
 struct OutOf<C, decltype((void)sizeof(typename C::Out))> { typedef typename C::Out type; };
 
+constexpr int kW4RMinK = 1792;  // measured: level at 1536, 7 % ahead at 2048, 13 % at 8192 (eight groups of 2048 rows)
+
 template <class C>
 __device__ __forceinline__ void run_tile(const typename C::Elem* Ap, int lda, int a_lim, const typename C::Elem* Bp,
                                          int ldb, int b_lim, int klen, typename OutOf<C>::type* Op, int ldo,
                                          typename C::Elem* smem, const SplitK& sk = SplitK()) {
   if constexpr (C::F32) gemm_tile_f32<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
-  else if constexpr (IsW4R<C>::value) gemm_tile_w4r<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
+  else if constexpr (IsW4R<C>::value) {
+    // The register-staged form has four 64-wide slabs to fill before it runs and pays for that on a short contraction:
+    // below kW4RMinK the 32-wide direct-to-LDS form of the same core takes the tile.
+    if (klen >= kW4RMinK) gemm_tile_w4r<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
+    else gemm_tile_w4<W4Cfg<C::BM, C::BN, true, true, 5>>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
+  }
   else if constexpr (IsW4<C>::value) gemm_tile_w4<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
   else if constexpr (C::MIXED) gemm_tile_pingpong_mixed<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
   else if constexpr (C::DLDS && C::PINGPONG) gemm_tile_pingpong<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
