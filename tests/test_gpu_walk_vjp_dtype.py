@@ -371,6 +371,41 @@ def test_short_group_row_tiles(k, split_k, trans_rhs):
         prev = y
 
 
+@pytest.mark.parametrize("split_k", [0, -1, 2])
+@pytest.mark.parametrize("n", [1728, 1792, 1800, 1864, 2048, 2584])
+def test_trans_rhs_long_contraction(n, split_k):
+    """gmm with trans_rhs on the four-wave variant around and above the contraction length (1792) from which its
+    register-staged form takes the tall tiles: whole and partial last 64-wide slabs, row tiles with 1 .. 256 live rows,
+    an empty group, a zero tail, a partial last column tile, with and without the K-split (whose pieces may fall back
+    under the threshold)."""
+    vid = [v.id for v in _capi.variants() if v.name.decode().startswith("w256")][0]
+    gs = np.array([300, 0, 17, 260, 123, 1, 640], np.int32)
+    g, k = gs.size, 520  # k: columns of the output here
+    m = int(gs.sum()) + 40
+    print(f"trans_rhs long contraction n={n} split_k={split_k}", flush=True)
+    lhs, rhs, dout, _, _ = util.make_case(n, m, k, n, g, 1.0, True, scale_rhs=True)
+    target_m = int(gs.sum())
+    d = util.bf16_dev(dout)
+    A = util.bf16_dev(rhs)  # [g, k, n]: with trans_rhs the contraction runs over n
+    gs_d = torch.from_numpy(gs).cuda()
+    plan = _capi.Plan(vid, 4, 0, 8, split_k=split_k)
+    ws = torch.empty(_capi.lib.rd_gmm_workspace_bytes(m, g, ctypes.byref(plan)), dtype=torch.uint8, device="cuda")
+    ws.fill_(0x5A)
+    ref = oracle.gmm(dout, rhs, gs, trans_rhs=True)
+    prev = None
+    for _ in range(2):
+        y = torch.full((m + 16, k), float("nan"), dtype=torch.bfloat16, device="cuda")
+        rc = _capi.lib.rd_gmm(_stream(), d.data_ptr(), A.data_ptr(), gs_d.data_ptr(), y.data_ptr(), m, n, k, g, 1,
+                              _capi.RD_DTYPE_BF16, ctypes.byref(plan), ws.data_ptr(), ws.numel())
+        assert rc == 0, _capi.lib.rd_last_error()
+        torch.cuda.synchronize()
+        assert torch.isnan(y[m:]).all() and not torch.isnan(y[:m]).any()
+        util.assert_close_rows(util.to_np(y[:m]), ref, target_m, util.BF16_EPS, "dlhs")
+        assert not torch.any(y[target_m:m])
+        assert prev is None or torch.equal(prev, y[:m])
+        prev = y[:m]
+
+
 # ---------------------------------------------------------------------------------------------------------------------
 # a slice of the groups (group_offset of jax.lax.ragged_dot; an expert-parallel rank's share of the weights)
 # ---------------------------------------------------------------------------------------------------------------------
