@@ -265,6 +265,25 @@ def test_decode_rows_kernel_many_groups(g, active, rows_each):
     assert not np.any(y[int(gs.sum()):])
 
 
+@pytest.mark.parametrize("k,n", [(520, 776), (2304, 200), (136, 2048)], ids=["k520-n776", "k2304-n200", "k136-n2048"])
+def test_decode_rows_kernel_wide_passes(k, n):
+    """More rows than groups: the whole-row streaming kernel takes up to 8 rows per pass (pairs of weight rows through
+    v_dot2_f32_bf16).  Every pass height 1 .. 8, groups that need two and three passes, empty groups, a zero tail, a
+    contraction longer than one staged segment, and one that is not a whole number of steps."""
+    from gpu_ragged_dot_amd import ops
+    print(f"decode rows kernel, wide passes k={k} n={n}", flush=True)
+    gs = np.array([0, 1, 2, 3, 4, 5, 6, 7, 8, 0, 9, 12, 16, 17, 0, 3], np.int32)
+    g, m = len(gs), int(gs.sum()) + 6
+    rng = np.random.default_rng(k + n)
+    lhs = oracle.round_to(rng.standard_normal((m, k)).astype(np.float32), "bfloat16")
+    rhs = oracle.round_to((rng.standard_normal((g, k, n)) / k ** 0.5).astype(np.float32), "bfloat16")
+    y = ops._gmm_fwd(util.bf16_dev(lhs), util.bf16_dev(rhs), torch.from_numpy(gs), 64, 64, 64, False, False, None,
+                     torch.float32, 512, plan=_capi.Plan(-1, 0, _capi.RD_DECODE_ROWS))
+    y = util.to_np(y)
+    util.assert_close_rows(y, oracle.gmm(lhs, rhs, gs), int(gs.sum()), util.BF16_EPS, "rows kernel, wide passes")
+    assert not np.any(y[int(gs.sum()):])
+
+
 # ---------------------------------------------------------------------------------------------------------------------
 # what the reference leaves undefined or never checks
 # ---------------------------------------------------------------------------------------------------------------------

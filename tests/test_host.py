@@ -120,8 +120,10 @@ def test_planner_choices():
     assert p.decode_nb == _capi.RD_DECODE_ROWS  # a few rows per expert -> streaming kernel (whole-row slices)
     p = planner.select_plan(_capi.OP_GMM_TRANS, 64, 2048, 768, 128)
     assert p.decode_nb == 0
-    p = planner.select_plan(_capi.OP_GMM, 256, 2048, 768, 128)
-    assert p.decode_nb == 0  # two rows per expert on average: some expert has more than a pass holds
+    p = planner.select_plan(_capi.OP_GMM, 512, 2048, 768, 128)
+    assert p.decode_nb == _capi.RD_DECODE_ROWS  # four rows per expert on average: still one pass of up to eight
+    p = planner.select_plan(_capi.OP_GMM, 1024, 2048, 768, 128)
+    assert p.decode_nb == 0
     p = planner.select_plan(_capi.OP_GMM, 16384, 4096, 14336, 8)
     assert vs[p.variant].tile_m == 256 and vs[p.variant].tile_n == 256
     p = planner.select_plan(_capi.OP_GMM, 16384, 4096, 14336, 8, block_m=128, block_k=64, block_n=128)
