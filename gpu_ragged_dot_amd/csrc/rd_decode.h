@@ -24,4 +24,9 @@ int launch_gmm_decode(hipStream_t s, const DecodeArgs& a, int nb);
 size_t gmm_rows_workspace_bytes(int m, int n, int pieces);
 int launch_gmm_rows(hipStream_t s, const DecodeArgs& a, int num_cus, void* workspace, size_t workspace_bytes);
 
+// The same for weights stored [g, n, k] (trans_rhs): the stream is cut along n, every piece yields complete sums, one
+// launch and no workspace.  DecodeArgs::A is then [g, n, k].  gmm_rows_t_fits: the shape can be served (k up to 8192).
+bool gmm_rows_t_fits(int m, int k, int n, int g);
+int launch_gmm_rows_t(hipStream_t s, const DecodeArgs& a, int num_cus);
+
 }  // namespace rd

@@ -558,6 +558,221 @@ __global__ __launch_bounds__(kThreads, 2) void gmm_rows_kernel(DecodeArgs p, Row
   }
 }
 
+// ---- trans_rhs: weights stored [g, n, k] --------------------------------------------------------------------------
+// Every weight row A[gi][j][:] is one contiguous run along the contraction index and yields one output column, so the
+// stream is cut along n: every non-empty expert gets the same number C of work-groups, each taking a contiguous block
+// of whole weight rows - and with them complete sums.  No partial sums, no workspace, one launch that writes y itself.
+// A wave takes one weight row at a time (64 lanes x 16 bytes = 1 KB per load, the four waves of a work-group four
+// consecutive rows); a lane multiplies its 8 contraction indices of the row with the same 8 of up to RMAX token rows
+// (both operands run along k, so pairs of bf16 meet in v_dot2_f32_bf16 as they are loaded), sums over its positions
+// along the row, and the 64 lanes' sums are added at the end of the row.
+constexpr int kTBlock = 4;        // weight rows a wave works on at a time: one read of the activations serves them all
+constexpr int kTDepth = 2;        // steps (of kTBlock 16-byte loads per lane) in flight
+constexpr int kTMaxLds = 64 * 1024;  // staged activations: RMAX rows x k (padded to 512) x 2 bytes
+
+// Sums of V values per lane over the 64 lanes of a wave.  Butterfly steps that halve the values as they go: in the step
+// with lane distance d a lane keeps one half of what it still holds, hands the other half to lane ^ d and adds what it
+// gets for its own half, so V - 1 exchanges (plus one per remaining step once a single value is left) replace the 6 V of
+// reducing every value by itself.  Returns the complete sum of value (lane >> (6 - log2 V)) & (V - 1).
+template <int V, int COUNT, int D>
+__device__ __forceinline__ float wave_sums_step(float (&v)[V], int lane) {
+  if constexpr (COUNT > 1) {
+    constexpr int HALF = COUNT / 2;
+    const bool upper = (lane & D) != 0;
+#pragma unroll
+    for (int i = 0; i < HALF; ++i) {
+      const float send = upper ? v[i] : v[i + HALF];
+      const float keep = upper ? v[i + HALF] : v[i];
+      v[i] = keep + __shfl_xor(send, D, 64);
+    }
+    return wave_sums_step<V, HALF, D / 2>(v, lane);
+  } else if constexpr (D >= 1) {
+    v[0] += __shfl_xor(v[0], D, 64);
+    return wave_sums_step<V, 1, D / 2>(v, lane);
+  } else {
+    return v[0];
+  }
+}
+template <int V>
+__device__ __forceinline__ float wave_sums(float (&v)[V], int lane) {
+  static_assert(V >= 1 && V <= 64 && (V & (V - 1)) == 0, "a power of two");
+  return wave_sums_step<V, V, 32>(v, lane);
+}
+
+template <int RMAX>
+__global__ __launch_bounds__(kThreads, 2) void gmm_rows_t_kernel(DecodeArgs p, int wgs) {
+  __shared__ int32_t wave_cnt[2][kThreads / 64];
+  __shared__ int32_t job[3];
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  u32x4_t* xs = reinterpret_cast<u32x4_t*>(smem_raw);  // [RMAX rows][chunk of 8 contraction indices] x 16 bytes
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+  // which experts are non-empty and where their rows start (as in gmm_rows_kernel)
+  auto scan_slab = [&](int base, int seen, int rows_seen, int& sz, int& rank, int& first_row, int& slab_act, int& slab_rows) {
+    const int e = base + tid;
+    sz = e < p.g ? imax(p.group_sizes[e], 0) : 0;
+    const unsigned long long m_act = __ballot(sz > 0);
+    const int before_in_wave = __popcll(m_act & ((1ull << lane) - 1ull));
+    int incl = sz;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) { const int up = __shfl_up(incl, d, 64); if (lane >= d) incl += up; }
+    __syncthreads();
+    if (lane == 63) { wave_cnt[0][wave] = __popcll(m_act); wave_cnt[1][wave] = incl; }
+    __syncthreads();
+    rank = seen + before_in_wave;
+    first_row = rows_seen + incl - sz;
+    slab_act = 0; slab_rows = 0;
+    for (int w2 = 0; w2 < kThreads / 64; ++w2) {
+      if (w2 < wave) { rank += wave_cnt[0][w2]; first_row += wave_cnt[1][w2]; }
+      slab_act += wave_cnt[0][w2]; slab_rows += wave_cnt[1][w2];
+    }
+  };
+  const bool one_slab = p.g <= kThreads;
+  int sz0 = 0, rank0 = 0, first0 = 0;
+  int n_act = 0, total = 0;
+  for (int base = 0; base < p.g; base += kThreads) {
+    int sz, rank, first_row, sa, sr;
+    scan_slab(base, n_act, total, sz, rank, first_row, sa, sr);
+    if (base == 0) { sz0 = sz; rank0 = rank; first0 = first_row; }
+    n_act += sa; total += sr;
+  }
+
+  // rows past sum(group_sizes) are zero: every work-group clears its share of them
+  {
+    const int t0 = imax(imin(total, p.m), 0);
+    const size_t words = (size_t)(p.m - t0) * p.n / 8;  // n % 8 == 0
+    u32x4_t* tail = reinterpret_cast<u32x4_t*>(p.y + (size_t)t0 * p.n);
+    for (size_t i = (size_t)blockIdx.x * kThreads + tid; i < words; i += (size_t)wgs * kThreads) tail[i] = u32x4_t{0, 0, 0, 0};
+  }
+  if (n_act == 0) return;
+  int C = imax(1, imin(wgs / n_act, p.n / kTBlock));  // a piece holds at least one block of weight rows
+  const int per = ((p.n + C - 1) / C + kTBlock - 1) / kTBlock * kTBlock;  // weight rows per piece (n % 8 == 0: whole blocks)
+  C = (p.n + per - 1) / per;                          // pieces that hold any
+  const int experts_at_a_time = wgs / C;
+  if ((int)blockIdx.x >= experts_at_a_time * C) return;
+  const int c = blockIdx.x % C;
+  const int j_begin = c * per, j_end = imin(p.n, j_begin + per);
+  const int chunks = p.k >> 3;                        // 16-byte chunks per weight row (k % 8 == 0)
+  const int npos = (chunks + 63) >> 6;                // loads per lane and weight row
+  const int r_stride = npos * 64;                     // staged entries per token row
+
+  for (int want = blockIdx.x / C; want < n_act; want += experts_at_a_time) {
+    __syncthreads();  // job free again
+    if (one_slab) {
+      if (sz0 > 0 && rank0 == want) { job[0] = tid; job[1] = first0; job[2] = sz0; }
+    } else {
+      int seen = 0, rows_seen = 0;
+      for (int base = 0; base < p.g; base += kThreads) {
+        int sz, rank, first_row, sa, sr;
+        scan_slab(base, seen, rows_seen, sz, rank, first_row, sa, sr);
+        if (sz > 0 && rank == want) { job[0] = base + tid; job[1] = first_row; job[2] = sz; }
+        seen += sa; rows_seen += sr;
+      }
+    }
+    __syncthreads();
+    const int gi = job[0], row0 = job[1];
+    const int rows = imin(job[2], p.m - row0);
+    if (rows <= 0) continue;
+    const bf16_bits* W = p.A + (size_t)gi * p.n * p.k;
+    // this wave's weight rows: blocks of kTBlock consecutive rows, block wave, wave + 4, ... of the piece (a piece is a
+    // whole number of blocks); its loads as one sequence of (block, position) steps of kTBlock loads each
+    const int blocks = (j_end - j_begin) / kTBlock;
+    const int my_blocks = wave < blocks ? (blocks - wave + 3) >> 2 : 0;
+    const int nsteps = my_blocks * npos;
+    // step s: position s % npos of block s / npos; the chunk is clamped to the row (the activations past k are zero)
+    auto load_step = [&](u32x4_t (&dst)[kTBlock], int s) {
+      const int sc = imin(s, nsteps - 1);
+      const int i = sc / npos, q = sc - i * npos;
+      const int ch = imin(q * 64 + lane, chunks - 1);
+      const uint32_t off = (uint32_t)(j_begin + kTBlock * (wave + 4 * i)) * (uint32_t)p.k + (uint32_t)ch * 8u;  // n * k < 2^31
+#pragma unroll
+      for (int b = 0; b < kTBlock; ++b)
+        dst[b] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(W + off + (uint32_t)b * (uint32_t)p.k));
+    };
+
+    for (int rc = 0; rc < rows; rc += RMAX) {
+      const int nr = imin(RMAX, rows - rc);
+      u32x4_t w[kTDepth][kTBlock];
+      if (nsteps > 0) {
+#pragma unroll
+        for (int u = 0; u < kTDepth; ++u) load_step(w[u], u);
+      }
+      __syncthreads();  // previous pass done with xs
+      // stage the activations: entry [row][chunk] = x[row][8 chunk .. 8 chunk + 7]; zero for rows past nr and for the
+      // chunks that pad the row to a whole number of positions (unconditional loads from clamped, valid addresses, four
+      // in flight per thread; masked afterwards)
+      for (int base = 0; base < r_stride * RMAX; base += kThreads * 4) {
+        u32x4_t v[4];
+#pragma unroll
+        for (int s2 = 0; s2 < 4; ++s2) {
+          const int idx = base + s2 * kThreads + tid;
+          const int r = imin(idx / r_stride, nr - 1), ch = imin(idx % r_stride, chunks - 1);
+          v[s2] = *reinterpret_cast<const u32x4_t*>(p.x + (size_t)(row0 + rc + r) * p.k + (size_t)ch * 8);
+        }
+#pragma unroll
+        for (int s2 = 0; s2 < 4; ++s2) {
+          const int idx = base + s2 * kThreads + tid;
+          const bool live = idx / r_stride < nr && idx % r_stride < chunks;
+          if (idx < r_stride * RMAX) xs[idx] = live ? v[s2] : u32x4_t{0, 0, 0, 0};
+        }
+      }
+      __syncthreads();
+      if (nsteps <= 0) continue;
+
+      float acc[kTBlock][RMAX];
+#pragma unroll
+      for (int b = 0; b < kTBlock; ++b)
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r) acc[b][r] = 0.f;
+      int q = 0, i = 0;  // position in the rows, block of this wave
+      for (int base = 0; base < nsteps; base += kTDepth) {
+#pragma unroll
+        for (int u = 0; u < kTDepth; ++u) {
+          if (base + u < nsteps) {  // uniform over the wave
+            const u32x4_t* xe = xs + (q * 64 + lane);
+#pragma unroll
+            for (int r = 0; r < RMAX; ++r) {
+              // one read of the token row's 8 activations serves the block's kTBlock weight rows.
+              // Scalars first: a bit cast applied to one element of a vector reads element 0 whatever the index.
+              const u32x4_t xv = xe[(size_t)r * r_stride];
+              const uint32_t x0 = xv[0], x1 = xv[1], x2 = xv[2], x3 = xv[3];
+#pragma unroll
+              for (int b = 0; b < kTBlock; ++b) {
+                const uint32_t w0 = w[u][b][0], w1 = w[u][b][1], w2 = w[u][b][2], w3 = w[u][b][3];
+                float a = acc[b][r];
+                a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w0), __builtin_bit_cast(bf16x2_t, x0), a, false);
+                a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w1), __builtin_bit_cast(bf16x2_t, x1), a, false);
+                a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w2), __builtin_bit_cast(bf16x2_t, x2), a, false);
+                a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w3), __builtin_bit_cast(bf16x2_t, x3), a, false);
+                acc[b][r] = a;
+              }
+            }
+            if (++q == npos) {
+              // end of the block's rows: the 64 lanes' sums of all kTBlock x RMAX values; every lane ends up with one of
+              // them, the first lane of each run of 64 / (kTBlock * RMAX) stores it
+              constexpr int V = kTBlock * RMAX, RUN = 64 / V;
+              float vals[V];
+#pragma unroll
+              for (int b = 0; b < kTBlock; ++b)
+#pragma unroll
+                for (int r = 0; r < RMAX; ++r) { vals[b * RMAX + r] = acc[b][r]; acc[b][r] = 0.f; }
+              const float mine = wave_sums<V>(vals, lane);
+              const int idx = lane / RUN;
+              const int b = idx / RMAX, r = idx - b * RMAX;
+              if (lane % RUN == 0 && r < nr)
+                p.y[(size_t)(row0 + rc + r) * p.n + (j_begin + kTBlock * (wave + 4 * i) + b)] = f32_to_bf16(mine);
+              q = 0; ++i;
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          load_step(w[u], base + kTDepth + u);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+  }
+}
+
 // y[row, :] = sum over the pieces of partials[row, piece, :] for rows below sum(group_sizes), zero above.
 // Work-group = (row, block of 256 columns); thread = (8 columns, one of 8 piece lanes).
 __global__ __launch_bounds__(kThreads) void gmm_rows_finish_kernel(DecodeArgs p, const RowsHeader* __restrict__ header,
@@ -650,6 +865,28 @@ int launch_gmm_rows(hipStream_t s, const DecodeArgs& a, int num_cus, void* works
   if (rc != hipSuccess) return rc;
   const int col_blocks = (a.n + 255) / 256;
   hipLaunchKernelGGL(gmm_rows_finish_kernel, dim3(a.m * col_blocks), dim3(kThreads), 0, s, a, header, partials);
+  return (int)hipGetLastError();
+}
+
+// trans_rhs: A is [g, n, k].  Needs k % 8 == 0, n % 8 == 0, n * k < 2^31 and rows-per-pass x k (padded to 512) x 2
+// bytes of LDS within kTMaxLds.  No workspace.
+bool gmm_rows_t_fits(int m, int k, int n, int g) {
+  (void)n;
+  const int kpad = (k + 511) & ~511;
+  return (long long)(m > g ? 8 : 4) * kpad * 2 <= kTMaxLds || (long long)4 * kpad * 2 <= kTMaxLds;
+}
+
+int launch_gmm_rows_t(hipStream_t s, const DecodeArgs& a, int num_cus) {
+  if (a.m <= 0 || a.n <= 0 || a.g <= 0) return hipSuccess;
+  if (a.n % 8 != 0 || a.k % 8 != 0 || a.k <= 0) return hipErrorInvalidValue;
+  const int kpad = (a.k + 511) & ~511;
+  const int wgs = 2 * (num_cus > 0 ? num_cus : 256);
+  // more than one row per group on average and room for them: 8 token rows per pass over the weights, else 4
+  const bool wide = a.m > a.g && (size_t)8 * kpad * 2 <= (size_t)kTMaxLds;
+  const size_t lds = (size_t)(wide ? 8 : 4) * kpad * 2;
+  if (lds > (size_t)kTMaxLds) return hipErrorInvalidValue;
+  if (wide) hipLaunchKernelGGL(gmm_rows_t_kernel<8>, dim3(wgs), dim3(kThreads), lds, s, a, wgs);
+  else hipLaunchKernelGGL(gmm_rows_t_kernel<4>, dim3(wgs), dim3(kThreads), lds, s, a, wgs);
   return (int)hipGetLastError();
 }
 

@@ -73,7 +73,8 @@ typedef struct rd_plan {
                   the product should equal what one XCD runs at a time (32 for the 256 x 256 tiles).  0 = default */
   int decode_nb; /* rd_gmm only, for a few rows per group: > 0 selects the streaming kernel that gives each work-group
                     this many columns (32, 64 or 128) of one expert; RD_DECODE_ROWS the one that gives it whole rows
-                    for a slice of the contraction range (fp32 partial sums in the workspace, n <= 2048) */
+                    for a slice of the contraction range (fp32 partial sums in the workspace, n <= 2048) or, with
+                    trans_rhs, whole weight rows of a slice of the columns (no partial sums, k <= 8192) */
   int split_k; /* rd_gmm only: 0 = when the tiles do not fill the device's last round and k >= 6400, cut those tiles'
                   contraction range over up to sqrt(k)/20 work-groups (fp32 partial sums in the workspace); n > 0 =
                   cut them over up to n (at most 8) whatever k is; -1 = never */
@@ -89,7 +90,8 @@ int rd_get_variant(int id, rd_variant_info* out /* host */);
  * For op 0 with m <= 4 g (and m <= 1024, n <= 2048) it selects the streaming kernel, which holds 4 rows of a group at a
  * time (8 when m > g) and streams the group's weights once per pass: right for a few rows per group, but if all m rows
  * belong to ONE group its weights are read m / 8 times.  The shape cannot tell; a caller who knows that its rows may
- * pile up in one group passes decode_nb = 0 with an explicit tile variant instead. */
+ * pile up in one group passes decode_nb = 0 with an explicit tile variant instead.  Op 1 (weights stored [g, n, k]) has a
+ * streaming kernel of its own under the same conditions and k <= 8192; it needs no workspace beyond the map's. */
 int rd_default_plan(int op, int m, int k, int n, int g, int dtype, rd_plan* out /* host */);
 
 /* ---- scheduling map --------------------------------------------------------------------------------------

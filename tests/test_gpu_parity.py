@@ -284,6 +284,61 @@ def test_decode_rows_kernel_wide_passes(k, n):
     assert not np.any(y[int(gs.sum()):])
 
 
+@pytest.mark.parametrize("case", ["decode-config", "long-groups-tail", "g600-sparse", "g300-two-rows", "wide-passes", "k8192", "n24"])
+def test_decode_rows_kernel_trans_rhs(case):
+    """Weights stored [g, n, k]: the streaming kernel that cuts every expert's weight rows into contiguous blocks along n
+    and writes y in one launch.  Default plan and explicit plan, 4 and 8 rows per pass, groups that need several passes,
+    empty groups, a zero tail, contraction lengths that are not a whole number of 512-element positions, more non-empty
+    groups than work-groups, fewer output columns than pieces."""
+    from gpu_ragged_dot_amd import ops
+    print(f"decode rows kernel, trans_rhs, {case}", flush=True)
+    rng = np.random.default_rng(len(case))
+    if case == "decode-config":
+        x, A, _, gs_t = workloads.make_inputs("decode")
+        lhs, rhs, gs = util.to_np(x), util.to_np(A), gs_t.cpu().numpy()
+    else:
+        k, n, gs = {
+            "long-groups-tail": (520, 200, np.array([0, 11, 1, 0, 9, 5], np.int32)),
+            "g600-sparse": (136, 72, None),
+            "g300-two-rows": (264, 40, None),
+            "wide-passes": (1032, 776, np.array([0, 1, 2, 3, 4, 5, 6, 7, 8, 0, 9, 12, 16, 17, 0, 3], np.int32)),
+            "k8192": (8192, 64, np.array([2, 0, 1, 3], np.int32)),
+            "n24": (2048, 24, np.array([1, 0, 4, 2, 0, 0, 1, 1], np.int32)),
+        }[case]
+        if gs is None:
+            g, active, rows_each = (600, 40, 1) if case == "g600-sparse" else (300, 299, 2)
+            gs = np.zeros(g, np.int32)
+            gs[rng.choice(g, active, replace=False)] = rows_each
+        g, m = len(gs), int(gs.sum()) + 5
+        lhs = oracle.round_to(rng.standard_normal((m, k)).astype(np.float32), "bfloat16")
+        rhs = oracle.round_to((rng.standard_normal((g, k, n)) / k ** 0.5).astype(np.float32), "bfloat16")
+    y_ref = oracle.gmm(lhs, rhs, gs)
+    rhs_t = np.ascontiguousarray(np.swapaxes(rhs, 1, 2))  # [g, n, k]
+    m = lhs.shape[0]
+    live = int(min(gs.sum(), m))
+    for plan in (_capi.Plan(-1, 0, _capi.RD_DECODE_ROWS), None):
+        y = ops._gmm_fwd(util.bf16_dev(lhs), util.bf16_dev(rhs_t), torch.from_numpy(gs), 64, 64, 64, True, False, None,
+                         torch.float32, 512, plan=plan)
+        y = util.to_np(y)
+        util.assert_close_rows(y, y_ref, live, util.BF16_EPS, f"trans_rhs rows kernel plan={plan}")
+        assert not np.any(y[live:])
+
+
+def test_decode_rows_kernel_trans_rhs_long_contraction_falls_back():
+    """A contraction too long for the streaming kernel's staged activations: refused when asked for by name, and the
+    default plan takes a tile kernel."""
+    from gpu_ragged_dot_amd import ops
+    k, n, gs = 8200, 16, np.array([1, 2], np.int32)
+    rng = np.random.default_rng(1)
+    lhs = oracle.round_to(rng.standard_normal((3, k)).astype(np.float32), "bfloat16")
+    rhs = oracle.round_to((rng.standard_normal((2, k, n)) / k ** 0.5).astype(np.float32), "bfloat16")
+    rhs_t = np.ascontiguousarray(np.swapaxes(rhs, 1, 2))
+    args = (util.bf16_dev(lhs), util.bf16_dev(rhs_t), torch.from_numpy(gs), 64, 64, 64, True, False, None, torch.float32, 512)
+    with pytest.raises(_capi.RaggedDotError):
+        ops._gmm_fwd(*args, plan=_capi.Plan(-1, 0, _capi.RD_DECODE_ROWS))
+    util.assert_close_rows(util.to_np(ops._gmm_fwd(*args)), oracle.gmm(lhs, rhs, gs), 3, util.BF16_EPS, "fallback")
+
+
 # ---------------------------------------------------------------------------------------------------------------------
 # what the reference leaves undefined or never checks
 # ---------------------------------------------------------------------------------------------------------------------

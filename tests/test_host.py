@@ -119,7 +119,9 @@ def test_planner_choices():
     p = planner.select_plan(_capi.OP_GMM, 64, 2048, 768, 128)
     assert p.decode_nb == _capi.RD_DECODE_ROWS  # a few rows per expert -> streaming kernel (whole-row slices)
     p = planner.select_plan(_capi.OP_GMM_TRANS, 64, 2048, 768, 128)
-    assert p.decode_nb == 0
+    assert p.decode_nb == _capi.RD_DECODE_ROWS  # weights stored [g, n, k] have a streaming kernel of their own
+    p = planner.select_plan(_capi.OP_GMM_TRANS, 64, 16384, 768, 128)
+    assert p.decode_nb == 0  # ... up to the contraction length whose activations it can stage
     p = planner.select_plan(_capi.OP_GMM, 512, 2048, 768, 128)
     assert p.decode_nb == _capi.RD_DECODE_ROWS  # four rows per expert on average: still one pass of up to eight
     p = planner.select_plan(_capi.OP_GMM, 1024, 2048, 768, 128)
