@@ -87,7 +87,7 @@ int rd_num_variants(void);
 int rd_get_variant(int id, rd_variant_info* out /* host */);
 
 /* The library's own shape-based choice (what variant = -1 resolves to); op: 0 gmm, 1 gmm trans_rhs, 2 tgmm.
- * For op 0 with m <= 4 g (and m <= 1024, n <= 2048) it selects the streaming kernel, which holds 4 rows of a group at a
+ * For op 0 with m <= 4 g (and m <= 1024, n <= 2048, min(g, m) * ceil(n / 256) <= 512) it selects the streaming kernel, which holds 4 rows of a group at a
  * time (8 when m > g) and streams the group's weights once per pass: right for a few rows per group, but if all m rows
  * belong to ONE group its weights are read m / 8 times.  The shape cannot tell; a caller who knows that its rows may
  * pile up in one group passes decode_nb = 0 with an explicit tile variant instead.  Op 1 (weights stored [g, n, k]) has a

@@ -126,6 +126,10 @@ def test_planner_choices():
     assert p.decode_nb == _capi.RD_DECODE_ROWS  # four rows per expert on average: still one pass of up to eight
     p = planner.select_plan(_capi.OP_GMM, 1024, 2048, 768, 128)
     assert p.decode_nb == 0
+    p = planner.select_plan(_capi.OP_GMM, 256, 7168, 2048, 256)
+    assert p.decode_nb == 0  # enough 256-column tiles for the tile kernels' streaming routines
+    p = planner.select_plan(_capi.OP_GMM, 64, 7168, 2048, 256)
+    assert p.decode_nb == _capi.RD_DECODE_ROWS
     p = planner.select_plan(_capi.OP_GMM, 16384, 4096, 14336, 8)
     assert vs[p.variant].tile_m == 256 and vs[p.variant].tile_n == 256
     p = planner.select_plan(_capi.OP_GMM, 16384, 4096, 14336, 8, block_m=128, block_k=64, block_n=128)
