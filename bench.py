@@ -9,7 +9,7 @@ workload (default: the Mixtral-8x7B-shaped forward+backward).  Unless --only is 
              roofline and cpu_baseline of its own;
   "context": what the same box does with a dense bf16 GEMM of the Mixtral forward's size (torch.matmul, on N(0,1)
              data and on zeros), a sustained (>= 2 s) loop of the headline step, a bare read of the decode shape's
-             bytes, and the CPU model.
+             bytes, the decode shape with its weights stored [g, n, k] (trans_rhs), and the CPU model.
 """
 
 import argparse
@@ -237,6 +237,22 @@ def measure(name, steps, warmup, torch, sustained_seconds=0.0, headline=False):
                             "median_ms_per_step": statistics.median(batches), "min_ms_per_step": min(batches)}
     if name == "decode":
         out["bare_stream"] = bare_stream(copies, abytes["weights_read"], torch)
+        # the same experts with their weights stored [g, n, k] (trans_rhs): context, not the metric's configuration
+        copies_t = [a.transpose(1, 2).contiguous() for a in copies]
+        del copies[1:]
+
+        def fwd_t():
+            a = copies_t[state["i"] % len(copies_t)]
+            state["i"] += 1
+            return ops._gmm_fwd(x, a, gs, **hp, trans_rhs=True)
+
+        for _ in range(max(warmup, 6)):
+            fwd_t()
+        ms_t = _event_ms(fwd_t, max(steps, 60), torch)
+        out["trans_rhs"] = {"what": "same shape, weights stored [g, n, k] (trans_rhs=True): one launch, no workspace",
+                            "us": ms_t * 1e3, "GB/s": abytes["weights_read"] / (ms_t * 1e-3) / 1e9,
+                            "plan": _plan_text(planner.select_plan(1, w.m, w.k, w.n, w.g), planner)}
+        del copies_t
     del x, A, dout, copies
     torch.cuda.empty_cache()
     return out
@@ -423,7 +439,8 @@ def main():
             configs[other] = c
         out["configs"] = configs
         out["context"] = {"dense_gemm": dense_gemm_context(torch), "sustained_headline_step": out.pop("sustained", None),
-                          "decode_bare_stream": configs["decode"].pop("bare_stream", None), "cpu": cpu_model(),
+                          "decode_bare_stream": configs["decode"].pop("bare_stream", None),
+                          "decode_trans_rhs": configs["decode"].pop("trans_rhs", None), "cpu": cpu_model(),
                           "device": torch.cuda.get_device_name(0)}
     print(json.dumps(out))
 
