@@ -3,11 +3,13 @@
 // rows, so the matrix cores are pointless and HBM bandwidth is everything.  No scheduling-map kernel runs first:
 // every work-group finds its group's row range itself from the group sizes.
 //
-// Two ways of cutting the stream into work-groups:
+// Three ways of cutting the stream into work-groups:
 //  * gmm_decode_kernel<NB>: work-group (group gi, column block jb) streams A[gi][:, jb*NB .. +NB) over the whole
 //    contraction range and writes y itself - one launch, no workspace;
 //  * gmm_rows_kernel: work-group (non-empty group, slice of the contraction range) streams whole rows of A[gi] - equal
-//    contiguous blocks - and leaves fp32 partial sums for gmm_rows_finish_kernel (second half of this file).
+//    contiguous blocks - and leaves fp32 partial sums for gmm_rows_finish_kernel;
+//  * gmm_rows_t_kernel, for weights stored [g, n, k] (trans_rhs): work-group (non-empty group, block of weight rows =
+//    output columns) - equal contiguous blocks again, but with complete sums: one launch, no workspace.
 // Both hold a few rows of x at a time in LDS (4; the whole-row kernel also has a form with 8), accumulate in fp32 on the
 // vector ALU and reduce across lanes at the end.
 #include "rd_common.h"
@@ -871,9 +873,9 @@ int launch_gmm_rows(hipStream_t s, const DecodeArgs& a, int num_cus, void* works
 // trans_rhs: A is [g, n, k].  Needs k % 8 == 0, n % 8 == 0, n * k < 2^31 and rows-per-pass x k (padded to 512) x 2
 // bytes of LDS within kTMaxLds.  No workspace.
 bool gmm_rows_t_fits(int m, int k, int n, int g) {
-  (void)n;
-  const int kpad = (k + 511) & ~511;
-  return (long long)(m > g ? 8 : 4) * kpad * 2 <= kTMaxLds || (long long)4 * kpad * 2 <= kTMaxLds;
+  (void)m; (void)n; (void)g;  // only the contraction length decides: 4 token rows of it must fit in LDS
+  const long long kpad = ((long long)k + 511) & ~511ll;
+  return k > 0 && 4 * kpad * 2 <= kTMaxLds;
 }
 
 int launch_gmm_rows_t(hipStream_t s, const DecodeArgs& a, int num_cus) {
