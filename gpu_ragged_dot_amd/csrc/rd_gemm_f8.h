@@ -1,0 +1,167 @@
+// float8 (OCP e4m3fn) operands on the float8 matrix-core instruction, for the product whose two operands both run along
+// the contraction index (gmm with trans_rhs: x[m, k] and A[g, n, k]).  Same structure as the direct-to-LDS core of
+// rd_gemm_dlds.h - a ring of K-slabs filled by buffer_load ... lds, one barrier per slab, the accumulators stored
+// through LDS as bf16 - with one-byte elements: a slab is 64 or 128 contraction indices deep (64- or 128-byte rows, the
+// geometry of a 32- or 64-deep bf16 slab, so the same loader and chunk permutation serve it), a lane's fragment is 8
+// consecutive bytes of its row (one ds_read_b64), and v_mfma_f32_32x32x16_fp8_fp8 multiplies them with fp32 accumulation.  Every e4m3
+// product is exact in fp32, so the result is what the bf16 path gives for the same values up to the order of the
+// additions.  Half the bytes of bf16 per operand element: what counts on the memory-bound shapes.
+// Needs 16-byte row pitches: k % 16 == 0.
+#pragma once
+#include "rd_gemm_dlds.h"
+
+namespace rd {
+
+// BK: contraction indices (= bytes) per slab row, 64 or 128.  128 makes every load cover whole 128-byte lines, which is
+// what a memory-bound tile wants; 64 halves the slab, which is what lets a 256 x 256 tile keep four of them.
+// B_AUX: cache policy of the B operand's loads (kCachePolicyStream: weights read once, not kept in L2).
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int STAGES_, int BK_ = 64, int B_AUX_ = 0>
+struct F8Cfg {
+  typedef fp8_bits Elem;
+  typedef bf16_bits Out;
+  static constexpr bool F32 = false, F8DIRECT = true;
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
+  static constexpr int B_AUX = B_AUX_;
+  static_assert(BK == 64 || BK == 128, "contraction slab");
+  static constexpr bool A_KMAJOR = true, B_KMAJOR = true, VEC = true, DLDS = true, PINGPONG = false, MIXED = false,
+                        SPLITK = false;
+  static constexpr int NW = WAVES_M * WAVES_N;
+  static constexpr int NT = 64 * NW;
+  static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  static constexpr int TM = WM / 32, TN = WN / 32;
+  static constexpr int KSTEPS = BK / 16;
+  static constexpr int TARGET_WGS = (TM * TN * 16 <= 64) ? (NW >= 8 ? 2 : 3) : 1;
+  static constexpr int WAVES_PER_EU = (NW / 4) * TARGET_WGS;
+  static constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
+  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int EPI_PITCH = WN * 2 + 16;
+  static constexpr int EPI_BYTES = NW * WM * EPI_PITCH;
+  static constexpr int RING_BYTES = STAGES * STAGE_BYTES;
+  static constexpr int LDS_BYTES = RING_BYTES > EPI_BYTES ? RING_BYTES : EPI_BYTES;
+  static_assert(BM % 64 == 0 && BN % 64 == 0 && BM % (32 * WAVES_M) == 0 && BN % (32 * WAVES_N) == 0, "tile shape");
+  static_assert(STAGES >= 2 && LDS_BYTES <= 160 * 1024, "LDS budget");
+};
+
+template <class C, class = void>
+struct IsF8Direct { static constexpr bool value = false; };
+template <class C>
+struct IsF8Direct<C, decltype((void)C::F8DIRECT)> { static constexpr bool value = true; };
+
+// Per-lane LDS byte offsets of the 8-byte fragments of a K-major float8 slab: [rows][BK bytes] with the 16-byte chunks of
+// a row permuted as the loader of a bf16 slab of the same row length leaves them - chunk c of row r at position
+// c ^ ((r >> 2) & 3) for 64-byte rows, c ^ ((r >> 1) & 7) for 128-byte rows.
+template <int BK>
+struct F8FragReader {
+  static constexpr int KSTEPS = BK / 16;
+  int addr[KSTEPS];
+  __device__ __forceinline__ void init(int row0, int lane) {
+    const int r = lane & 31;
+    const int sw = BK == 128 ? ((r >> 1) & 7) : ((r >> 2) & 3);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) addr[ks] = (row0 + r) * BK + ((ks ^ sw) << 4) + (lane >> 5) * 8;
+  }
+  // lane l: row (l & 31) of 32-row block `tile`, contraction bytes 16 ks + 8 (l >> 5) .. + 7
+  __device__ __forceinline__ long read(const unsigned char* region, int tile, int ks) const {
+    return *reinterpret_cast<const long*>(region + addr[ks] + tile * 32 * BK);
+  }
+};
+
+// Same contract as gemm_tile_dlds(): Ap/Bp point at the tile's first row and first contraction index, lda/ldb are row
+// pitches in elements (multiples of 16), a_lim/b_lim the live rows of each operand, klen the contraction length
+// (a multiple of 16).
+template <class C>
+__device__ __forceinline__ void gemm_tile_f8(const fp8_bits* __restrict__ Ap, int lda, int a_lim,
+                                             const fp8_bits* __restrict__ Bp, int ldb, int b_lim, int klen,
+                                             bf16_bits* __restrict__ Op, int ldo, fp8_bits* smem_) {
+  unsigned char* smem = reinterpret_cast<unsigned char*>(smem_);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;
+
+  // the byte mover of a bf16 slab of the same row length: pitches and lengths in 2-byte units
+  constexpr int BK2 = C::BK / 2;
+  typedef DldsLoader<C::BM, BK2, C::NW, true> LdA;
+  typedef DldsLoader<C::BN, BK2, C::NW, true, C::B_AUX> LdB;
+  LdA la; LdB lb;
+  const int klen2 = klen >> 1;
+  la.init(reinterpret_cast<const bf16_bits*>(Ap), lda >> 1, a_lim, klen2, wave, lane);
+  lb.init(reinterpret_cast<const bf16_bits*>(Bp), ldb >> 1, b_lim, klen2, wave, lane);
+  F8FragReader<C::BK> fra, frb;
+  fra.init(wm * C::WM, lane);
+  frb.init(wn * C::WN, lane);
+  const bool patch_live = wm * C::WM < a_lim && wn * C::WN < b_lim;
+
+  f32x16_t acc[C::TM][C::TN];
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  const int nk = (klen + C::BK - 1) / C::BK;
+  constexpr int L = LdA::PER + LdB::PER;  // loads per thread per K-step
+
+  auto issue_loads = [&](int step, int first, int count) {
+    unsigned char* st = smem + (step % C::STAGES) * C::STAGE_BYTES;
+    const int k0 = step * BK2;  // in 2-byte units, like klen2
+    const bool tail = k0 + BK2 > klen2;
+    __amdgpu_buffer_rsrc_t ra_ = la.resource(), rb_ = lb.resource();
+#pragma unroll
+    for (int q = first; q < first + count; ++q) {
+      if (q < LdA::PER) {
+        if (tail) la.template issue<true>(ra_, st, wave, q, k0, klen2);
+        else la.template issue<false>(ra_, st, wave, q, k0, klen2);
+      } else {
+        if (tail) lb.template issue<true>(rb_, st + C::A_BYTES, wave, q - LdA::PER, k0, klen2);
+        else lb.template issue<false>(rb_, st + C::A_BYTES, wave, q - LdA::PER, k0, klen2);
+      }
+    }
+  };
+
+#pragma unroll
+  for (int s = 0; s < C::STAGES - 1; ++s)
+    if (s < nk) { issue_loads(s, 0, L); la.advance(); lb.advance(); }
+
+  for (int kt = 0; kt < nk; ++kt) {
+    if (kt + C::STAGES - 2 < nk) wait_vmcnt<(C::STAGES - 2) * L>(); else wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();  // every wave's part of slab kt is in LDS, and slab kt-1 is no longer being read
+    const bool more = kt + C::STAGES - 1 < nk;
+    const unsigned char* ra = smem + (kt % C::STAGES) * C::STAGE_BYTES;
+    const unsigned char* rb = ra + C::A_BYTES;
+    long fa[2][C::TM], fb[2][C::TN];
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i) fa[0][i] = fra.read(ra, i, 0);
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) fb[0][j] = frb.read(rb, j, 0);
+#pragma unroll
+    for (int ks = 0; ks < C::KSTEPS; ++ks) {
+      const int cur = ks & 1, nxt = cur ^ 1;
+      if (ks + 1 < C::KSTEPS) {
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i) fa[nxt][i] = fra.read(ra, i, ks + 1);
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) fb[nxt][j] = frb.read(rb, j, ks + 1);
+      }
+      if (more) {
+        const int first = (L * ks) / C::KSTEPS, last = (L * (ks + 1)) / C::KSTEPS;
+        issue_loads(kt + C::STAGES - 1, first, last - first);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (patch_live) {
+#pragma unroll
+        for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+          for (int j = 0; j < C::TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (more) { la.advance(); lb.advance(); }
+  }
+
+  __builtin_amdgcn_s_barrier();  // the ring is no longer read by any wave
+  store_accumulators<C>(acc, wm, wn, wave, lane, a_lim, b_lim, Op, ldo, smem);
+}
+
+}  // namespace rd

@@ -3,6 +3,7 @@
 #pragma once
 #include "rd_gemm_dlds.h"
 #include "rd_gemm_f32.h"
+#include "rd_gemm_f8.h"
 #include "rd_gemm_w4.h"
 #include "rd_gemm_w4r.h"
 #include "rd_gemm_pp.h"
@@ -74,6 +75,7 @@ __device__ __forceinline__ void run_tile(const typename C::Elem* Ap, int lda, in
                                          int ldb, int b_lim, int klen, typename OutOf<C>::type* Op, int ldo,
                                          typename C::Elem* smem, const SplitK& sk = SplitK()) {
   if constexpr (C::F32) gemm_tile_f32<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
+  else if constexpr (IsF8Direct<C>::value) gemm_tile_f8<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
   else if constexpr (IsW4R<C>::value) {
     // The register-staged form has four 64-wide slabs to fill before it runs and pays for that on a short contraction:
     // below kW4RMinK the 32-wide direct-to-LDS form of the same core takes the tile.
@@ -248,6 +250,18 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
         return;
       }
     }
+    if constexpr (IsF8Direct<C>::value) {
+      // float8: the same split between a group's only row tile, when it is short, and the tall tiles - the short tile
+      // is a stream over its 256 weight rows in 128-deep slabs of whole cache lines (three 40 KB slabs in the ring), read past L2
+      if constexpr (C::BM > kShortRows && C::NT == 256 && C::BN == 256) {
+        typedef F8Cfg<kShortRows, C::BN, 1, 4, 3, 128, kCachePolicyStream> S;
+        static_assert(S::LDS_BYTES <= C::LDS_BYTES && S::NT == C::NT, "the short routine runs in the tall one's launch");
+        if (rows <= kShortRows && it == 0) {
+          gemm_tile_f8<S>(Ap, p.k, rows, Bp, p.k, cols, klen, Op, p.n, smem);
+          return;
+        }
+      }
+    }
     run_tile<C>(Ap, p.k, rows, Bp, TRANS_RHS ? p.k : p.n, cols, klen, Op, p.n, smem, sk);
   } else {
     // Rows past sum(group_sizes) are defined to be zero.  The map never uses more than
@@ -309,7 +323,7 @@ struct TileVariant {
   int dlds;    // 1: direct-to-LDS core (byte extents of one tile's operand window must stay below 2 GiB)
   int stages;  // LDS ring depth
   int splitk;  // 1: the gmm kernels can cut the last round of tiles along K (needs partials in the workspace)
-  gmm_launch_fn gmm_nn, gmm_nt;
+  gmm_launch_fn gmm_nn, gmm_nt;  // null: the shape has no kernel for that product
   tgmm_launch_fn tgmm;
 };
 

@@ -24,7 +24,11 @@
 #endif
 
 namespace rd {
-#if RD_F32 == 3
+#if RD_F32 == 3 && RD_DLDS
+// float8 e4m3fn arrays on the float8 matrix-core instruction, direct-to-LDS: the product with two K-major operands only
+#define RD_ONLY_NT 1
+typedef F8Cfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, RD_STAGES> CfgNT;
+#elif RD_F32 == 3
 // float8 e4m3fn arrays, widened to bf16 on the way into LDS, bf16 matrix cores, bf16 out
 typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, /*A K-major*/ true, /*B K-major*/ false, RD_VEC != 0, fp8_bits> CfgNN;
 typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, true, true, RD_VEC != 0, fp8_bits> CfgNT;
@@ -65,6 +69,10 @@ extern "C" const rd::TileVariant* RD_CAT(rd_variant_, RD_NAME)() {
   static const rd::TileVariant v = {
       RD_STR(RD_NAME), RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, RD_VEC, /*dtype: RD_DTYPE_* */ RD_F32, RD_DLDS != 0, RD_STAGES,
       /*splitk*/ RD_DLDS != 0 && !RD_F32,
+#ifdef RD_ONLY_NT
+      nullptr, &rd::launch_gmm<rd::CfgNT, true>, nullptr};
+#else
       &rd::launch_gmm<rd::CfgNN, false>, &rd::launch_gmm<rd::CfgNT, true>, &rd::launch_tgmm<rd::CfgTN>};
+#endif
   return &v;
 }
