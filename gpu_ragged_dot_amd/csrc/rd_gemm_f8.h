@@ -1,12 +1,16 @@
-// float8 (OCP e4m3fn) operands on the float8 matrix-core instruction, for the product whose two operands both run along
-// the contraction index (gmm with trans_rhs: x[m, k] and A[g, n, k]).  Same structure as the direct-to-LDS core of
+// float8 (OCP e4m3fn) operands on the float8 matrix-core instruction.  Same structure as the direct-to-LDS core of
 // rd_gemm_dlds.h - a ring of K-slabs filled by buffer_load ... lds, one barrier per slab, the accumulators stored
-// through LDS as bf16 - with one-byte elements: a slab is 64 or 128 contraction indices deep (64- or 128-byte rows, the
-// geometry of a 32- or 64-deep bf16 slab, so the same loader and chunk permutation serve it), a lane's fragment is 8
-// consecutive bytes of its row (one ds_read_b64), and v_mfma_f32_32x32x16_fp8_fp8 multiplies them with fp32 accumulation.  Every e4m3
-// product is exact in fp32, so the result is what the bf16 path gives for the same values up to the order of the
-// additions.  Half the bytes of bf16 per operand element: what counts on the memory-bound shapes.
-// Needs 16-byte row pitches: k % 16 == 0.
+// through LDS as bf16 - with one-byte elements.  The bytes are moved by the loader of a bf16 slab with the same row
+// length (so its chunk permutations apply unchanged):
+//   K-major operand  (contraction index contiguous): slab [rows][BK bytes], BK = 64 or 128; a lane's fragment is 8
+//                    consecutive bytes of its row, one ds_read_b64;
+//   MN-major operand (weights [k, n], both operands of tgmm): slab [BK][rows bytes]; the 8-bit transposing LDS read
+//                    (ds_read_b64_tr_b8: 16 lanes read an 8 x 16 byte block, lane i gets the 8 bytes of column i) hands a
+//                    lane the 8 contraction-consecutive bytes of its column.
+// v_mfma_f32_32x32x16_fp8_fp8 multiplies the fragments with fp32 accumulation.  Every e4m3 product is exact in fp32, so
+// the result is what the bf16 path gives for the same values up to the order of the additions.  Half the bytes of bf16
+// per operand element: what counts on the memory-bound shapes.  Needs 16-byte row pitches (k % 16 == 0, and n % 16 == 0
+// where n is a row pitch).
 #pragma once
 #include "rd_gemm_dlds.h"
 
@@ -15,7 +19,8 @@ namespace rd {
 // BK: contraction indices (= bytes) per slab row, 64 or 128.  128 makes every load cover whole 128-byte lines, which is
 // what a memory-bound tile wants; 64 halves the slab, which is what lets a 256 x 256 tile keep four of them.
 // B_AUX: cache policy of the B operand's loads (kCachePolicyStream: weights read once, not kept in L2).
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int STAGES_, int BK_ = 64, int B_AUX_ = 0>
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int STAGES_, int BK_ = 64, int B_AUX_ = 0, bool A_KMAJOR_ = true,
+          bool B_KMAJOR_ = true>
 struct F8Cfg {
   typedef fp8_bits Elem;
   typedef bf16_bits Out;
@@ -23,7 +28,9 @@ struct F8Cfg {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
   static constexpr int B_AUX = B_AUX_;
   static_assert(BK == 64 || BK == 128, "contraction slab");
-  static constexpr bool A_KMAJOR = true, B_KMAJOR = true, VEC = true, DLDS = true, PINGPONG = false, MIXED = false,
+  // an MN-major slab row holds the operand's whole tile extent, and its chunk permutation needs 16 chunks (256 bytes)
+  static_assert((A_KMAJOR_ || BM_ % 256 == 0) && (B_KMAJOR_ || BN_ % 256 == 0), "MN-major tile extents");
+  static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = true, DLDS = true, PINGPONG = false, MIXED = false,
                         SPLITK = false;
   static constexpr int NW = WAVES_M * WAVES_N;
   static constexpr int NT = 64 * NW;
@@ -66,9 +73,45 @@ struct F8FragReader {
   }
 };
 
-// Same contract as gemm_tile_dlds(): Ap/Bp point at the tile's first row and first contraction index, lda/ldb are row
-// pitches in elements (multiples of 16), a_lim/b_lim the live rows of each operand, klen the contraction length
-// (a multiple of 16).
+// MN-major float8 slab [BK][ROW_BYTES] with chunk c of contraction row kk at position c ^ ((kk & 3) << 2) (the loader of
+// an MN-major bf16 slab).  A 16-lane group q reads the 8 x 16 byte block of contraction rows 8 (q >> 1) .. + 7 and
+// columns 16 (q & 1) .. + 15 of its 32-column block: lane i supplies the address of row (i >> 1), bytes 8 (i & 1) .. + 7,
+// and receives the 8 contraction-consecutive bytes of column i.
+template <int ROW_BYTES, int TILES>
+struct F8FragReaderT {
+  int addr[TILES];
+  __device__ __forceinline__ void init(int col0, int lane) {
+    const int q = lane >> 4, i = lane & 15;
+    const int row = 8 * (q >> 1) + (i >> 1);
+    const int s = ((i >> 1) & 3) << 2;
+#pragma unroll
+    for (int j = 0; j < TILES; ++j) {
+      const int chunk = ((col0 >> 4) + 2 * j + (q & 1)) ^ s;
+      addr[j] = row * ROW_BYTES + (chunk << 4) + (i & 1) * 8;
+    }
+  }
+  __device__ __forceinline__ long read(const unsigned char* region, int tile, int ks) const {
+    typedef int v2i_t __attribute__((ext_vector_type(2)));
+    typedef __attribute__((address_space(3))) v2i_t* lds_v2i_ptr;
+    const v2i_t v = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(region + addr[tile] + ks * 16 * ROW_BYTES));
+    return __builtin_bit_cast(long, v);
+  }
+};
+
+// The reader of one operand, whichever way it is laid out.
+template <int T, int BK, int TILES, bool KMAJOR>
+struct F8Frag {
+  F8FragReader<BK> km;
+  F8FragReaderT<T, TILES> mn;
+  __device__ __forceinline__ void init(int idx0, int lane) { if (KMAJOR) km.init(idx0, lane); else mn.init(idx0, lane); }
+  __device__ __forceinline__ long read(const unsigned char* region, int tile, int ks) const {
+    return KMAJOR ? km.read(region, tile, ks) : mn.read(region, tile, ks);
+  }
+};
+
+// Same contract as gemm_tile_dlds(): Ap/Bp point at the tile's first row (K-major) or column (MN-major) and first
+// contraction index, lda/ldb are row pitches in elements (multiples of 16), a_lim/b_lim the live rows / columns of each
+// operand, klen the contraction length (a multiple of 16 for K-major operands).
 template <class C>
 __device__ __forceinline__ void gemm_tile_f8(const fp8_bits* __restrict__ Ap, int lda, int a_lim,
                                              const fp8_bits* __restrict__ Bp, int ldb, int b_lim, int klen,
@@ -78,15 +121,17 @@ __device__ __forceinline__ void gemm_tile_f8(const fp8_bits* __restrict__ Ap, in
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;
 
-  // the byte mover of a bf16 slab of the same row length: pitches and lengths in 2-byte units
+  // The byte mover of a bf16 slab of the same row length.  K-major: [T rows][BK / 2 elements], pitch, tail length and
+  // slab advance in 2-byte units.  MN-major: [BK rows][T / 2 elements], extent limit in 2-byte units, whole rows of k.
   constexpr int BK2 = C::BK / 2;
-  typedef DldsLoader<C::BM, BK2, C::NW, true> LdA;
-  typedef DldsLoader<C::BN, BK2, C::NW, true, C::B_AUX> LdB;
+  typedef DldsLoader<C::A_KMAJOR ? C::BM : C::BM / 2, C::A_KMAJOR ? BK2 : C::BK, C::NW, C::A_KMAJOR> LdA;
+  typedef DldsLoader<C::B_KMAJOR ? C::BN : C::BN / 2, C::B_KMAJOR ? BK2 : C::BK, C::NW, C::B_KMAJOR, C::B_AUX> LdB;
   LdA la; LdB lb;
   const int klen2 = klen >> 1;
-  la.init(reinterpret_cast<const bf16_bits*>(Ap), lda >> 1, a_lim, klen2, wave, lane);
-  lb.init(reinterpret_cast<const bf16_bits*>(Bp), ldb >> 1, b_lim, klen2, wave, lane);
-  F8FragReader<C::BK> fra, frb;
+  la.init(reinterpret_cast<const bf16_bits*>(Ap), lda >> 1, C::A_KMAJOR ? a_lim : (a_lim + 1) >> 1, C::A_KMAJOR ? klen2 : klen, wave, lane);
+  lb.init(reinterpret_cast<const bf16_bits*>(Bp), ldb >> 1, C::B_KMAJOR ? b_lim : (b_lim + 1) >> 1, C::B_KMAJOR ? klen2 : klen, wave, lane);
+  F8Frag<C::BM, C::BK, C::TM, C::A_KMAJOR> fra;
+  F8Frag<C::BN, C::BK, C::TN, C::B_KMAJOR> frb;
   fra.init(wm * C::WM, lane);
   frb.init(wn * C::WN, lane);
   const bool patch_live = wm * C::WM < a_lim && wn * C::WN < b_lim;
@@ -104,7 +149,9 @@ __device__ __forceinline__ void gemm_tile_f8(const fp8_bits* __restrict__ Ap, in
 
   auto issue_loads = [&](int step, int first, int count) {
     unsigned char* st = smem + (step % C::STAGES) * C::STAGE_BYTES;
-    const int k0 = step * BK2;  // in 2-byte units, like klen2
+    // The tail test only concerns K-major operands (whose counts are in 2-byte units, like klen2): an MN-major slab's
+    // rows past the contraction length lie outside the loader's buffer and read as zeros by themselves.
+    const int k0 = step * BK2;
     const bool tail = k0 + BK2 > klen2;
     __amdgpu_buffer_rsrc_t ra_ = la.resource(), rb_ = lb.resource();
 #pragma unroll

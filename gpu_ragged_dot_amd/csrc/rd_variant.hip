@@ -25,9 +25,15 @@
 
 namespace rd {
 #if RD_F32 == 3 && RD_DLDS
-// float8 e4m3fn arrays on the float8 matrix-core instruction, direct-to-LDS: the product with two K-major operands only
-#define RD_ONLY_NT 1
-typedef F8Cfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, RD_STAGES> CfgNT;
+// float8 e4m3fn arrays on the float8 matrix-core instruction, direct-to-LDS (rd_gemm_f8.h).  tgmm reads x^T as an
+// MN-major operand, whose slab rows span the tile's rows: only for tile heights that are multiples of 256.
+typedef F8Cfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, RD_STAGES, 64, 0, /*A K-major*/ true, /*B K-major*/ false> CfgNN;
+typedef F8Cfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, RD_STAGES, 64, 0, true, true> CfgNT;
+#if RD_BM % 256 == 0
+typedef F8Cfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, RD_STAGES, 64, 0, false, false> CfgTN;
+#else
+#define RD_NO_TGMM 1
+#endif
 #elif RD_F32 == 3
 // float8 e4m3fn arrays, widened to bf16 on the way into LDS, bf16 matrix cores, bf16 out
 typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, /*A K-major*/ true, /*B K-major*/ false, RD_VEC != 0, fp8_bits> CfgNN;
@@ -69,8 +75,8 @@ extern "C" const rd::TileVariant* RD_CAT(rd_variant_, RD_NAME)() {
   static const rd::TileVariant v = {
       RD_STR(RD_NAME), RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, RD_VEC, /*dtype: RD_DTYPE_* */ RD_F32, RD_DLDS != 0, RD_STAGES,
       /*splitk*/ RD_DLDS != 0 && !RD_F32,
-#ifdef RD_ONLY_NT
-      nullptr, &rd::launch_gmm<rd::CfgNT, true>, nullptr};
+#ifdef RD_NO_TGMM
+      &rd::launch_gmm<rd::CfgNN, false>, &rd::launch_gmm<rd::CfgNT, true>, nullptr};
 #else
       &rd::launch_gmm<rd::CfgNN, false>, &rd::launch_gmm<rd::CfgNT, true>, &rd::launch_tgmm<rd::CfgTN>};
 #endif

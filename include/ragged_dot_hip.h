@@ -35,8 +35,9 @@ extern "C" {
  * product of two bfloat16 values is exact in fp32, and the accumulation is fp32 either way.)
  * RD_DTYPE_F8E4M3_BF16: both operands (x and A of rd_gmm, x and dy of rd_tgmm) are float8 e4m3fn bytes (the OCP format:
  * bias 7, no infinities, 0x7f / 0xff are NaN), the output is bfloat16 - jax.lax.ragged_dot on float8 operands with
- * preferred_element_type = bfloat16; the reference itself has no float8 path.  With trans_rhs and k % 16 == 0 the bytes
- * go to the float8 matrix-core instruction as they are (fp32 accumulation); otherwise they are widened to bfloat16 as
+ * preferred_element_type = bfloat16; the reference itself has no float8 path.  With 16-byte row pitches (k % 16 == 0,
+ * and n % 16 == 0 unless trans_rhs) the bytes go to the float8 matrix-core instruction as they are (fp32
+ * accumulation); otherwise they are widened to bfloat16 as
  * they are loaded (exact: every e4m3 value is a bfloat16 value) and multiplied on the bf16 matrix cores.  Either way the
  * result is that of an exact-product fp32-accumulating float8 multiply; what float8 buys is half the bytes read, not a
  * higher matrix-core rate.  Tile kernels only (no streaming kernel for a few rows per group, no K-split). */

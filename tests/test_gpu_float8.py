@@ -89,7 +89,7 @@ def test_float8_products_against_the_oracle(shape):
     assert not np.any(util.to_np(dA)[gs == 0])
 
 
-@pytest.mark.parametrize("shape", [(1030, 264, 392, 5), (515, 99, 131, 3), (1300, 272, 520, 4), (700, 1040, 264, 9)],
+@pytest.mark.parametrize("shape", [(1030, 264, 392, 5), (515, 99, 131, 3), (1300, 272, 520, 4), (700, 1040, 264, 9), (900, 528, 400, 6)],
                          ids=lambda s: "m%d_k%d_n%d_g%d" % s)
 def test_float8_every_tile_shape(shape):
     """Each tile shape compiled for float8 operands, forced through the plan (the 8-byte-chunk ones only where the
@@ -113,8 +113,9 @@ def test_float8_every_tile_shape(shape):
         print("float8 tile", v.name.decode(), shape, flush=True)
         plan = _capi.Plan(v.id)
         ws = torch.empty(max(_capi.lib.rd_gmm_workspace_bytes(m, g, ctypes.byref(plan)), 256), dtype=torch.uint8, device="cuda")
-        # the direct-to-LDS float8 shapes have the trans_rhs kernel only
-        for trans_rhs, rhs in (((1, At),) if v.direct_to_lds else ((0, A), (1, At))):
+        # the direct-to-LDS float8 shapes need 16-byte row pitches: n % 16 == 0 too when n is one (weights [g, k, n], tgmm)
+        direct_needs_n16 = v.direct_to_lds and n % 16 != 0
+        for trans_rhs, rhs in (((1, At),) if direct_needs_n16 else ((0, A), (1, At))):
             y = torch.full((m + guard, n), float("nan"), dtype=torch.bfloat16, device="cuda")
             rc = _capi.lib.rd_gmm(torch.cuda.current_stream().cuda_stream, x.data_ptr(), rhs.data_ptr(), gs_d.data_ptr(),
                                   y.data_ptr(), m, k, n, g, trans_rhs, _capi.RD_DTYPE_F8E4M3_BF16, ctypes.byref(plan),
@@ -125,12 +126,13 @@ def test_float8_every_tile_shape(shape):
             assert np.isnan(got[m:]).all() and not np.isnan(got[:m]).any()
             util.assert_close_rows(got[:m], y_ref, target_m, util.BF16_EPS, f"gmm {v.name.decode()} trans_rhs={trans_rhs}")
             assert not np.any(got[target_m:m])
-        if v.direct_to_lds:
+        if direct_needs_n16:
             y = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
             rc = _capi.lib.rd_gmm(torch.cuda.current_stream().cuda_stream, x.data_ptr(), A.data_ptr(), gs_d.data_ptr(),
                                   y.data_ptr(), m, k, n, g, 0, _capi.RD_DTYPE_F8E4M3_BF16, ctypes.byref(plan),
                                   ws.data_ptr(), ws.numel())
             assert rc == _capi.RD_ERR_UNSUPPORTED  # refused by name, not mis-run
+        if direct_needs_n16 or (v.direct_to_lds and v.tile_m % 256):  # (x^T as an operand: 256-row tiles only)
             with pytest.raises(_capi.RaggedDotError):
                 ops._tgmm_fwd(x, d, gs_d, **HP, plan=plan)
             ran += 1
