@@ -1,17 +1,17 @@
-// float8 (OCP e4m3fn) operands on the float8 matrix-core instruction.  Same structure as the direct-to-LDS core of
-// rd_gemm_dlds.h - a ring of K-slabs filled by buffer_load ... lds, one barrier per slab, the accumulators stored
+// float8 (OCP e4m3fn) operands on the float8 matrix-core instruction v_mfma_f32_32x32x64_f8f6f4 (64 contraction indices
+// per instruction, fp32 accumulation, twice the rate of the bf16 instruction).  Same structure as the direct-to-LDS core
+// of rd_gemm_dlds.h - a ring of K-slabs filled by buffer_load ... lds, one barrier per slab, the accumulators stored
 // through LDS as bf16 - with one-byte elements.  The bytes are moved by the loader of a bf16 slab with the same row
 // length (so its chunk permutations apply unchanged):
-//   K-major operand  (contraction index contiguous): slab [rows][BK bytes], BK = 64 or 128; a lane's fragment is 8
-//                    consecutive bytes of its row, one ds_read_b64;
+//   K-major operand  (contraction index contiguous): slab [rows][BK bytes], BK = 64 or 128; a lane's fragment is 32
+//                    consecutive bytes of its row, two ds_read_b128;
 //   MN-major operand (weights [k, n], both operands of tgmm): slab [BK][rows bytes]; the 8-bit transposing LDS read
 //                    (ds_read_b64_tr_b8: 16 lanes read an 8 x 16 byte block, lane i gets the 8 bytes of column i) hands a
-//                    lane the 8 contraction-consecutive bytes of its column.
-// v_mfma_f32_32x32x16_fp8_fp8 multiplies the fragments with fp32 accumulation.  Every e4m3 product is exact in fp32, so
-// the result is what the bf16 path gives for the same values up to the order of the additions.  Half the bytes of bf16
-// per operand element: what counts on the memory-bound shapes.  Needs 16-byte row pitches (k % 16 == 0, and n % 16 == 0
-// where n is a row pitch).
+//                    lane 8 contraction-consecutive bytes of its column, four of them a fragment.
+// Every e4m3 product is exact in fp32, so the result is what the bf16 path gives for the same values up to the order of
+// the additions.  Needs 16-byte row pitches (k % 16 == 0, and n % 16 == 0 where n is a row pitch).
 #pragma once
+#include <type_traits>
 #include "rd_gemm_dlds.h"
 
 namespace rd {
@@ -36,7 +36,7 @@ struct F8Cfg {
   static constexpr int NT = 64 * NW;
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   static constexpr int TM = WM / 32, TN = WN / 32;
-  static constexpr int KSTEPS = BK / 16;
+  static constexpr int KSTEPS = BK / 64;  // matrix-core steps per slab
   static constexpr int TARGET_WGS = (TM * TN * 16 <= 64) ? (NW >= 8 ? 2 : 3) : 1;
   static constexpr int WAVES_PER_EU = (NW / 4) * TARGET_WGS;
   static constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
@@ -54,35 +54,40 @@ struct IsF8Direct { static constexpr bool value = false; };
 template <class C>
 struct IsF8Direct<C, decltype((void)C::F8DIRECT)> { static constexpr bool value = true; };
 
-// Per-lane LDS byte offsets of the 8-byte fragments of a K-major float8 slab: [rows][BK bytes] with the 16-byte chunks of
-// a row permuted as the loader of a bf16 slab of the same row length leaves them - chunk c of row r at position
-// c ^ ((r >> 2) & 3) for 64-byte rows, c ^ ((r >> 1) & 7) for 128-byte rows.
+// Fragments of v_mfma_f32_32x32x64_f8f6f4: lane l feeds row / column (l & 31) and the 32 contraction bytes
+// 32 (l >> 5) .. + 31 of a 64-deep step, in byte order - whatever the instruction's own numbering of them is, both
+// operands are read the same way, so equal positions hold equal contraction indices.
+typedef int i32x8_t __attribute__((ext_vector_type(8)));
+// K-major slab [rows][BK bytes], the 16-byte chunks of a row permuted as the loader of a bf16 slab of the same row length
+// leaves them (chunk c of row r at position c ^ ((r >> 2) & 3) for 64-byte rows, c ^ ((r >> 1) & 7) for 128-byte rows):
+// two 16-byte chunks of the lane's row.
 template <int BK>
 struct F8FragReader {
-  static constexpr int KSTEPS = BK / 16;
-  int addr[KSTEPS];
+  int addr[BK / 64][2];
   __device__ __forceinline__ void init(int row0, int lane) {
     const int r = lane & 31;
     const int sw = BK == 128 ? ((r >> 1) & 7) : ((r >> 2) & 3);
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) addr[ks] = (row0 + r) * BK + ((ks ^ sw) << 4) + (lane >> 5) * 8;
+    for (int ws = 0; ws < BK / 64; ++ws)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) addr[ws][h] = (row0 + r) * BK + (((4 * ws + 2 * (lane >> 5) + h) ^ sw) << 4);
   }
-  // lane l: row (l & 31) of 32-row block `tile`, contraction bytes 16 ks + 8 (l >> 5) .. + 7
-  __device__ __forceinline__ long read(const unsigned char* region, int tile, int ks) const {
-    return *reinterpret_cast<const long*>(region + addr[ks] + tile * 32 * BK);
+  __device__ __forceinline__ i32x8_t read(const unsigned char* region, int tile, int ws) const {
+    const u32x4_t lo = *reinterpret_cast<const u32x4_t*>(region + addr[ws][0] + tile * 32 * BK);
+    const u32x4_t hi = *reinterpret_cast<const u32x4_t*>(region + addr[ws][1] + tile * 32 * BK);
+    return i32x8_t{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
   }
 };
-
-// MN-major float8 slab [BK][ROW_BYTES] with chunk c of contraction row kk at position c ^ ((kk & 3) << 2) (the loader of
-// an MN-major bf16 slab).  A 16-lane group q reads the 8 x 16 byte block of contraction rows 8 (q >> 1) .. + 7 and
-// columns 16 (q & 1) .. + 15 of its 32-column block: lane i supplies the address of row (i >> 1), bytes 8 (i & 1) .. + 7,
-// and receives the 8 contraction-consecutive bytes of column i.
+// MN-major slab [BK][ROW_BYTES], chunk c of contraction row kk at position c ^ ((kk & 3) << 2) (the loader of an MN-major
+// bf16 slab): four 8-bit transposing reads (ds_read_b64_tr_b8) of 8 contraction rows each.  In one such read a 16-lane
+// group fetches an 8 x 16 byte block - lane i supplies the address of row (i >> 1), bytes 8 (i & 1) .. + 7 - and lane i
+// receives the 8 contraction-consecutive bytes of column i.
 template <int ROW_BYTES, int TILES>
 struct F8FragReaderT {
   int addr[TILES];
   __device__ __forceinline__ void init(int col0, int lane) {
     const int q = lane >> 4, i = lane & 15;
-    const int row = 8 * (q >> 1) + (i >> 1);
+    const int row = 32 * (q >> 1) + (i >> 1);
     const int s = ((i >> 1) & 3) << 2;
 #pragma unroll
     for (int j = 0; j < TILES; ++j) {
@@ -90,22 +95,24 @@ struct F8FragReaderT {
       addr[j] = row * ROW_BYTES + (chunk << 4) + (i & 1) * 8;
     }
   }
-  __device__ __forceinline__ long read(const unsigned char* region, int tile, int ks) const {
+  __device__ __forceinline__ i32x8_t read(const unsigned char* region, int tile, int ws) const {
     typedef int v2i_t __attribute__((ext_vector_type(2)));
     typedef __attribute__((address_space(3))) v2i_t* lds_v2i_ptr;
-    const v2i_t v = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(region + addr[tile] + ks * 16 * ROW_BYTES));
-    return __builtin_bit_cast(long, v);
+    const unsigned char* p = region + addr[tile] + ws * 64 * ROW_BYTES;
+    const v2i_t a = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(p));
+    const v2i_t b = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(p + 8 * ROW_BYTES));
+    const v2i_t c = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(p + 16 * ROW_BYTES));
+    const v2i_t d = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_ptr)(p + 24 * ROW_BYTES));
+    return i32x8_t{a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
   }
 };
-
-// The reader of one operand, whichever way it is laid out.
 template <int T, int BK, int TILES, bool KMAJOR>
 struct F8Frag {
   F8FragReader<BK> km;
   F8FragReaderT<T, TILES> mn;
   __device__ __forceinline__ void init(int idx0, int lane) { if (KMAJOR) km.init(idx0, lane); else mn.init(idx0, lane); }
-  __device__ __forceinline__ long read(const unsigned char* region, int tile, int ks) const {
-    return KMAJOR ? km.read(region, tile, ks) : mn.read(region, tile, ks);
+  __device__ __forceinline__ i32x8_t read(const unsigned char* region, int tile, int ws) const {
+    return KMAJOR ? km.read(region, tile, ws) : mn.read(region, tile, ws);
   }
 };
 
@@ -176,22 +183,25 @@ __device__ __forceinline__ void gemm_tile_f8(const fp8_bits* __restrict__ Ap, in
     const bool more = kt + C::STAGES - 1 < nk;
     const unsigned char* ra = smem + (kt % C::STAGES) * C::STAGE_BYTES;
     const unsigned char* rb = ra + C::A_BYTES;
-    long fa[2][C::TM], fb[2][C::TN];
+    // Fragments of step ks + 1 are fetched from LDS while the matrix core works on step ks, and the loads of the slab
+    // STAGES - 1 ahead are issued a few at a time between the steps.
+    constexpr int NSTEP = C::KSTEPS;
+    i32x8_t fa[2][C::TM], fb[2][C::TN];
 #pragma unroll
     for (int i = 0; i < C::TM; ++i) fa[0][i] = fra.read(ra, i, 0);
 #pragma unroll
     for (int j = 0; j < C::TN; ++j) fb[0][j] = frb.read(rb, j, 0);
 #pragma unroll
-    for (int ks = 0; ks < C::KSTEPS; ++ks) {
+    for (int ks = 0; ks < NSTEP; ++ks) {
       const int cur = ks & 1, nxt = cur ^ 1;
-      if (ks + 1 < C::KSTEPS) {
+      if (ks + 1 < NSTEP) {
 #pragma unroll
         for (int i = 0; i < C::TM; ++i) fa[nxt][i] = fra.read(ra, i, ks + 1);
 #pragma unroll
         for (int j = 0; j < C::TN; ++j) fb[nxt][j] = frb.read(rb, j, ks + 1);
       }
       if (more) {
-        const int first = (L * ks) / C::KSTEPS, last = (L * (ks + 1)) / C::KSTEPS;
+        const int first = (L * ks) / NSTEP, last = (L * (ks + 1)) / NSTEP;
         issue_loads(kt + C::STAGES - 1, first, last - first);
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -199,8 +209,8 @@ __device__ __forceinline__ void gemm_tile_f8(const fp8_bits* __restrict__ Ap, in
 #pragma unroll
         for (int i = 0; i < C::TM; ++i)
 #pragma unroll
-          for (int j = 0; j < C::TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
+          for (int j = 0; j < C::TN; ++j)  // both formats e4m3, no block scales: the plain 32x32x64 instruction
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0, 0, 0, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
     }

@@ -250,20 +250,6 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
         return;
       }
     }
-    if constexpr (IsF8Direct<C>::value) {
-      // float8: the same split between a group's only row tile, when it is short, and the tall tiles - the short tile
-      // is a stream over its 256 columns of the group's weights, read past L2
-      if constexpr (C::BM > kShortRows && C::NT == 256 && C::BN == 256) {
-        // weights along k: 128-deep slabs of whole cache lines, three 40 KB slabs; weights across k: 64-deep, six of 20 KB
-        typedef typename std::conditional<C::B_KMAJOR, F8Cfg<kShortRows, C::BN, 1, 4, 3, 128, kCachePolicyStream, true, true>,
-                                          F8Cfg<kShortRows, C::BN, 1, 4, 6, 64, kCachePolicyStream, true, false>>::type S;
-        static_assert(S::LDS_BYTES <= C::LDS_BYTES && S::NT == C::NT, "the short routine runs in the tall one's launch");
-        if (rows <= kShortRows && it == 0) {
-          gemm_tile_f8<S>(Ap, p.k, rows, Bp, TRANS_RHS ? p.k : p.n, cols, klen, Op, p.n, smem);
-          return;
-        }
-      }
-    }
     run_tile<C>(Ap, p.k, rows, Bp, TRANS_RHS ? p.k : p.n, cols, klen, Op, p.n, smem, sk);
   } else {
     // Rows past sum(group_sizes) are defined to be zero.  The map never uses more than
