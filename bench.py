@@ -9,7 +9,8 @@ workload (default: the Mixtral-8x7B-shaped forward+backward).  Unless --only is 
              roofline and cpu_baseline of its own;
   "context": what the same box does with a dense bf16 GEMM of the Mixtral forward's size (torch.matmul, on N(0,1)
              data and on zeros), a sustained (>= 2 s) loop of the headline step, a bare read of the decode shape's
-             bytes, the decode shape with its weights stored [g, n, k] (trans_rhs), and the CPU model.
+             bytes, the decode shape with its weights stored [g, n, k] (trans_rhs), the Mixtral-shaped products on float8
+             operands, and the CPU model.
 """
 
 import argparse
@@ -311,6 +312,32 @@ def dense_gemm_context(torch):
                     "dout.W^T (dlhs layout), x^T.dout (drhs layout)", **out}
 
 
+def float8_context(torch):
+    """The Mixtral-shaped products with float8 e4m3fn operands (bf16 out, fp32 accumulation): forward products only - the
+    library has no float8 VJP - so this is context beside the bf16 metric, not a configuration of it."""
+    from gpu_ragged_dot_amd import ops, workloads
+
+    name = "mixtral_fwd_bwd"
+    x, A, dout, gs = workloads.make_inputs(name)
+    w = workloads.WORKLOADS[name]
+    hp = dict(block_m=64, block_k=64, block_n=64, interpret=False, compute_dtype=None, acc_dtype=torch.float32, chunk_m=512)
+    x8, A8, d8 = (t.to(torch.float8_e4m3fn) for t in (x, A, dout))
+    del x, A, dout
+    parts = (("gmm", lambda: ops._gmm_fwd(x8, A8, gs, **hp, trans_rhs=False)),
+             ("gmm_trans_rhs", lambda: ops._gmm_fwd(d8, A8, gs, **hp, trans_rhs=True)),
+             ("tgmm", lambda: ops._tgmm_fwd(x8, d8, gs, **hp)))
+    flops = workloads.flops(name) / 3
+    out = {"what": "m16384 k4096 n14336 g8, float8 e4m3fn operands, bf16 out: x.W[g], dout.W[g]^T, x^T.dout per group"}
+    for pname, fn in parts:
+        for _ in range(3):
+            fn()
+        ms = _event_ms(fn, 20, torch)
+        out[pname] = {"ms": ms, "TFLOP/s": flops / (ms * 1e-3) / 1e12, "frac_of_fp8_mfma_peak": flops / (ms * 1e-3) / 1e12 / 5033.2}
+    del x8, A8, d8
+    torch.cuda.empty_cache()
+    return out
+
+
 def bench_routing(args, torch):
     """The caller's side of the DeepSeek-V3 shaped workload: 4096 tokens x top-8 of 256 experts.  One step = route
     the (token, choice) pairs, gather the 7168-wide activations into expert order, and sum a 2048-wide product back
@@ -440,7 +467,8 @@ def main():
         out["configs"] = configs
         out["context"] = {"dense_gemm": dense_gemm_context(torch), "sustained_headline_step": out.pop("sustained", None),
                           "decode_bare_stream": configs["decode"].pop("bare_stream", None),
-                          "decode_trans_rhs": configs["decode"].pop("trans_rhs", None), "cpu": cpu_model(),
+                          "decode_trans_rhs": configs["decode"].pop("trans_rhs", None),
+                          "float8_mixtral_products": float8_context(torch), "cpu": cpu_model(),
                           "device": torch.cuda.get_device_name(0)}
     print(json.dumps(out))
 
