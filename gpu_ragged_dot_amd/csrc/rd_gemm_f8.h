@@ -20,7 +20,7 @@ namespace rd {
 // what a memory-bound tile wants; 64 halves the slab, which is what lets a 256 x 256 tile keep four of them.
 // B_AUX: cache policy of the B operand's loads (kCachePolicyStream: weights read once, not kept in L2).
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int STAGES_, int BK_ = 64, int B_AUX_ = 0, bool A_KMAJOR_ = true,
-          bool B_KMAJOR_ = true>
+          bool B_KMAJOR_ = true, bool PINGPONG_ = false>
 struct F8Cfg {
   typedef fp8_bits Elem;
   typedef bf16_bits Out;
@@ -30,7 +30,7 @@ struct F8Cfg {
   static_assert(BK == 64 || BK == 128, "contraction slab");
   // an MN-major slab row holds the operand's whole tile extent, and its chunk permutation needs 16 chunks (256 bytes)
   static_assert((A_KMAJOR_ || BM_ % 256 == 0) && (B_KMAJOR_ || BN_ % 256 == 0), "MN-major tile extents");
-  static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = true, DLDS = true, PINGPONG = false, MIXED = false,
+  static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = true, DLDS = true, PINGPONG = PINGPONG_, MIXED = false,
                         SPLITK = false;
   static constexpr int NW = WAVES_M * WAVES_N;
   static constexpr int NT = 64 * NW;
@@ -47,6 +47,7 @@ struct F8Cfg {
   static constexpr int LDS_BYTES = RING_BYTES > EPI_BYTES ? RING_BYTES : EPI_BYTES;
   static_assert(BM % 64 == 0 && BN % 64 == 0 && BM % (32 * WAVES_M) == 0 && BN % (32 * WAVES_N) == 0, "tile shape");
   static_assert(STAGES >= 2 && LDS_BYTES <= 160 * 1024, "LDS budget");
+  static_assert(!PINGPONG_ || (NW == 8 && WAVES_M_ == 2 && STAGES_ >= 3 && BK_ == 64), "ping-pong runs two groups of four waves");
 };
 
 template <class C, class = void>
@@ -218,6 +219,105 @@ __device__ __forceinline__ void gemm_tile_f8(const fp8_bits* __restrict__ Ap, in
   }
 
   __builtin_amdgcn_s_barrier();  // the ring is no longer read by any wave
+  store_accumulators<C>(acc, wm, wn, wave, lane, a_lim, b_lim, Op, ldo, smem);
+}
+
+// The ping-pong schedule of rd_gemm_dlds.h on the float8 fragments: the eight waves form two groups of four (one wave of
+// each per SIMD) that alternate, half a period apart, between a memory phase (the slab's fragments LDS -> registers,
+// the wave's share of the direct loads of a later slab) and a compute phase (matrix-core instructions only), one
+// work-group barrier per phase.
+template <class C>
+__device__ __forceinline__ void gemm_tile_f8_pingpong(const fp8_bits* __restrict__ Ap, int lda, int a_lim,
+                                                      const fp8_bits* __restrict__ Bp, int ldb, int b_lim, int klen,
+                                                      bf16_bits* __restrict__ Op, int ldo, fp8_bits* smem_) {
+  unsigned char* smem = reinterpret_cast<unsigned char*>(smem_);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;
+  const int group = wave >> 2;
+
+  constexpr int BK2 = C::BK / 2;
+  typedef DldsLoader<C::A_KMAJOR ? C::BM : C::BM / 2, C::A_KMAJOR ? BK2 : C::BK, C::NW, C::A_KMAJOR> LdA;
+  typedef DldsLoader<C::B_KMAJOR ? C::BN : C::BN / 2, C::B_KMAJOR ? BK2 : C::BK, C::NW, C::B_KMAJOR, C::B_AUX> LdB;
+  LdA la; LdB lb;
+  const int klen2 = klen >> 1;
+  la.init(reinterpret_cast<const bf16_bits*>(Ap), lda >> 1, C::A_KMAJOR ? a_lim : (a_lim + 1) >> 1, C::A_KMAJOR ? klen2 : klen, wave, lane);
+  lb.init(reinterpret_cast<const bf16_bits*>(Bp), ldb >> 1, C::B_KMAJOR ? b_lim : (b_lim + 1) >> 1, C::B_KMAJOR ? klen2 : klen, wave, lane);
+  F8Frag<C::BM, C::BK, C::TM, C::A_KMAJOR> fra;
+  F8Frag<C::BN, C::BK, C::TN, C::B_KMAJOR> frb;
+  fra.init(wm * C::WM, lane);
+  frb.init(wn * C::WN, lane);
+  const bool patch_live = wm * C::WM < a_lim && wn * C::WN < b_lim;
+
+  f32x16_t acc[C::TM][C::TN];
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  const int nk = (klen + C::BK - 1) / C::BK;
+  constexpr int L = LdA::PER + LdB::PER;
+
+  auto issue_slab = [&](int step) {
+    unsigned char* st = smem + (step % C::STAGES) * C::STAGE_BYTES;
+    const int k0 = step * BK2;
+    const bool tail = k0 + BK2 > klen2;
+    __amdgpu_buffer_rsrc_t ra_ = la.resource(), rb_ = lb.resource();
+#pragma unroll
+    for (int q = 0; q < LdA::PER; ++q) {
+      if (tail) la.template issue<true>(ra_, st, wave, q, k0, klen2);
+      else la.template issue<false>(ra_, st, wave, q, k0, klen2);
+    }
+#pragma unroll
+    for (int q = 0; q < LdB::PER; ++q) {
+      if (tail) lb.template issue<true>(rb_, st + C::A_BYTES, wave, q, k0, klen2);
+      else lb.template issue<false>(rb_, st + C::A_BYTES, wave, q, k0, klen2);
+    }
+    la.advance();
+    lb.advance();
+  };
+
+#pragma unroll
+  for (int s = 0; s < C::STAGES - 1; ++s)
+    if (s < nk) issue_slab(s);
+  if (C::STAGES - 1 <= nk) wait_vmcnt<(C::STAGES - 2) * L>(); else wait_vmcnt<0>();
+  __builtin_amdgcn_s_barrier();
+  if (group == 1) __builtin_amdgcn_s_barrier();
+
+  for (int kt = 0; kt < nk; ++kt) {
+    // ---- memory phase ---------------------------------------------------------------------------------------------
+    const unsigned char* ra = smem + (kt % C::STAGES) * C::STAGE_BYTES;
+    const unsigned char* rb = ra + C::A_BYTES;
+    i32x8_t fa[C::TM], fb[C::TN];
+    if (patch_live) {
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i) fa[i] = fra.read(ra, i, 0);
+#pragma unroll
+      for (int j = 0; j < C::TN; ++j) fb[j] = frb.read(rb, j, 0);
+    }
+    if (kt + C::STAGES - 1 < nk) issue_slab(kt + C::STAGES - 1);
+    if (kt + C::STAGES - 1 < nk) wait_vmcnt<(C::STAGES - 2) * L>(); else wait_vmcnt<0>();
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- compute phase --------------------------------------------------------------------------------------------
+    __builtin_amdgcn_s_setprio(1);
+    if (patch_live) {
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[j], fa[i], acc[i][j], 0, 0, 0, 0, 0, 0);
+    }
+    __builtin_amdgcn_s_setprio(0);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (group == 0) __builtin_amdgcn_s_barrier();
   store_accumulators<C>(acc, wm, wn, wave, lane, a_lim, b_lim, Op, ldo, smem);
 }
 

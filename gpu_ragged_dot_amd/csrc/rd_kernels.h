@@ -75,7 +75,10 @@ __device__ __forceinline__ void run_tile(const typename C::Elem* Ap, int lda, in
                                          int ldb, int b_lim, int klen, typename OutOf<C>::type* Op, int ldo,
                                          typename C::Elem* smem, const SplitK& sk = SplitK()) {
   if constexpr (C::F32) gemm_tile_f32<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
-  else if constexpr (IsF8Direct<C>::value) gemm_tile_f8<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
+  else if constexpr (IsF8Direct<C>::value) {
+    if constexpr (C::PINGPONG) gemm_tile_f8_pingpong<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
+    else gemm_tile_f8<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
+  }
   else if constexpr (IsW4R<C>::value) {
     // The register-staged form has four 64-wide slabs to fill before it runs and pays for that on a short contraction:
     // below kW4RMinK the 32-wide direct-to-LDS form of the same core takes the tile.

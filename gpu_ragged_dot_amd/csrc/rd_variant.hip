@@ -27,10 +27,10 @@ namespace rd {
 #if RD_F32 == 3 && RD_DLDS
 // float8 e4m3fn arrays on the float8 matrix-core instruction, direct-to-LDS (rd_gemm_f8.h).  tgmm reads x^T as an
 // MN-major operand, whose slab rows span the tile's rows: only for tile heights that are multiples of 256.
-typedef F8Cfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, RD_STAGES, 64, 0, /*A K-major*/ true, /*B K-major*/ false> CfgNN;
-typedef F8Cfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, RD_STAGES, 64, 0, true, true> CfgNT;
+typedef F8Cfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, RD_STAGES, 64, 0, /*A K-major*/ true, /*B K-major*/ false, RD_PINGPONG != 0> CfgNN;
+typedef F8Cfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, RD_STAGES, 64, 0, true, true, RD_PINGPONG != 0> CfgNT;
 #if RD_BM % 256 == 0
-typedef F8Cfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, RD_STAGES, 64, 0, false, false> CfgTN;
+typedef F8Cfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, RD_STAGES, 64, 0, false, false, RD_PINGPONG != 0> CfgTN;
 #else
 #define RD_NO_TGMM 1
 #endif
