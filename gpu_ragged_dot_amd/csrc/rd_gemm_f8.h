@@ -31,7 +31,7 @@ struct F8Cfg {
   // an MN-major slab row holds the operand's whole tile extent, and its chunk permutation needs 16 chunks (256 bytes)
   static_assert((A_KMAJOR_ || BM_ % 256 == 0) && (B_KMAJOR_ || BN_ % 256 == 0), "MN-major tile extents");
   static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = true, DLDS = true, PINGPONG = PINGPONG_, MIXED = false,
-                        SPLITK = false;
+                        SPLITK = true;
   static constexpr int NW = WAVES_M * WAVES_N;
   static constexpr int NT = 64 * NW;
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
@@ -123,7 +123,8 @@ struct F8Frag {
 template <class C>
 __device__ __forceinline__ void gemm_tile_f8(const fp8_bits* __restrict__ Ap, int lda, int a_lim,
                                              const fp8_bits* __restrict__ Bp, int ldb, int b_lim, int klen,
-                                             bf16_bits* __restrict__ Op, int ldo, fp8_bits* smem_) {
+                                             bf16_bits* __restrict__ Op, int ldo, fp8_bits* smem_,
+                                             const SplitK& sk = SplitK()) {
   unsigned char* smem = reinterpret_cast<unsigned char*>(smem_);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -219,6 +220,7 @@ __device__ __forceinline__ void gemm_tile_f8(const fp8_bits* __restrict__ Ap, in
   }
 
   __builtin_amdgcn_s_barrier();  // the ring is no longer read by any wave
+  if (!splitk_combine<C>(acc, sk, tid, smem)) return;
   store_accumulators<C>(acc, wm, wn, wave, lane, a_lim, b_lim, Op, ldo, smem);
 }
 
@@ -229,7 +231,8 @@ __device__ __forceinline__ void gemm_tile_f8(const fp8_bits* __restrict__ Ap, in
 template <class C>
 __device__ __forceinline__ void gemm_tile_f8_pingpong(const fp8_bits* __restrict__ Ap, int lda, int a_lim,
                                                       const fp8_bits* __restrict__ Bp, int ldb, int b_lim, int klen,
-                                                      bf16_bits* __restrict__ Op, int ldo, fp8_bits* smem_) {
+                                                      bf16_bits* __restrict__ Op, int ldo, fp8_bits* smem_,
+                                                      const SplitK& sk = SplitK()) {
   unsigned char* smem = reinterpret_cast<unsigned char*>(smem_);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -318,6 +321,7 @@ __device__ __forceinline__ void gemm_tile_f8_pingpong(const fp8_bits* __restrict
     __builtin_amdgcn_sched_barrier(0);
   }
   if (group == 0) __builtin_amdgcn_s_barrier();
+  if (!splitk_combine<C>(acc, sk, tid, smem)) return;
   store_accumulators<C>(acc, wm, wn, wave, lane, a_lim, b_lim, Op, ldo, smem);
 }
 

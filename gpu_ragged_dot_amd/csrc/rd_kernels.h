@@ -76,8 +76,8 @@ __device__ __forceinline__ void run_tile(const typename C::Elem* Ap, int lda, in
                                          typename C::Elem* smem, const SplitK& sk = SplitK()) {
   if constexpr (C::F32) gemm_tile_f32<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
   else if constexpr (IsF8Direct<C>::value) {
-    if constexpr (C::PINGPONG) gemm_tile_f8_pingpong<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
-    else gemm_tile_f8<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem);
+    if constexpr (C::PINGPONG) gemm_tile_f8_pingpong<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
+    else gemm_tile_f8<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
   }
   else if constexpr (IsW4R<C>::value) {
     // The register-staged form has four 64-wide slabs to fill before it runs and pays for that on a short contraction:
@@ -121,7 +121,8 @@ struct SplitPlan {
 constexpr int kMaxSplitParts = 8;
 constexpr int kMinSplitK = 512;  // contraction elements a piece must keep
 
-__device__ __forceinline__ SplitPlan split_plan(int live, int k, int slots, int num_cus, int max_parts) {
+// k_cost: the contraction length in units of what a bf16 K loop spends per element (float8 operands: k / 2).
+__device__ __forceinline__ SplitPlan split_plan(int live, int k, int k_cost, int slots, int num_cus, int max_parts) {
   SplitPlan sp{live, 1, 0};
   if (slots <= 0 || live <= 0) return sp;
   const int first = (live / num_cus) * num_cus;
@@ -136,7 +137,7 @@ __device__ __forceinline__ SplitPlan split_plan(int live, int k, int slots, int 
     parts = imin(parts, max_parts);
   } else {
     int by_k = 1;
-    while ((by_k + 1) * (by_k + 1) * 400 <= k) ++by_k;
+    while ((by_k + 1) * (by_k + 1) * 400 <= k_cost) ++by_k;
     if (by_k < 4) return sp;
     parts = imin(parts, by_k);
   }
@@ -175,7 +176,7 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
   const int total = imin(uniform(*p.total_tiles), p.U);
   const int live = total * p.n_tiles;
   SplitPlan sp{live, 1, 0};
-  if constexpr (C::SPLITK) sp = split_plan(live, p.k, p.split_slots, p.num_cus, p.max_parts);
+  if constexpr (C::SPLITK) sp = split_plan(live, p.k, sizeof(E) == 1 ? p.k >> 1 : p.k, p.split_slots, p.num_cus, p.max_parts);
 
   int t;
   SplitK sk;

@@ -74,7 +74,7 @@ typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, false, false, RD_VE
 extern "C" const rd::TileVariant* RD_CAT(rd_variant_, RD_NAME)() {
   static const rd::TileVariant v = {
       RD_STR(RD_NAME), RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, RD_VEC, /*dtype: RD_DTYPE_* */ RD_F32, RD_DLDS != 0, RD_STAGES,
-      /*splitk*/ RD_DLDS != 0 && !RD_F32,
+      /*splitk*/ RD_DLDS != 0 && (!RD_F32 || RD_F32 == 3),
 #ifdef RD_NO_TGMM
       &rd::launch_gmm<rd::CfgNN, false>, &rd::launch_gmm<rd::CfgNT, true>, nullptr};
 #else

@@ -39,8 +39,9 @@ extern "C" {
  * and n % 16 == 0 unless trans_rhs) the bytes go to the float8 matrix-core instruction as they are (fp32
  * accumulation); otherwise they are widened to bfloat16 as
  * they are loaded (exact: every e4m3 value is a bfloat16 value) and multiplied on the bf16 matrix cores.  Either way the
- * result is that of an exact-product fp32-accumulating float8 multiply; what float8 buys is half the bytes read, not a
- * higher matrix-core rate.  Tile kernels only (no streaming kernel for a few rows per group, no K-split). */
+ * result is that of an exact-product fp32-accumulating float8 multiply; the first path has half the bytes to read and
+ * twice the matrix-core rate of bfloat16, the second only the former.  Tile kernels only (no streaming kernel for a few
+ * rows per group); the K-split of rd_plan.split_k on the first path only. */
 enum rd_dtype { RD_DTYPE_BF16 = 0, RD_DTYPE_F32 = 1, RD_DTYPE_F32_BF16 = 2, RD_DTYPE_F8E4M3_BF16 = 3 };
 
 #define RD_DECODE_ROWS (-1) /* rd_plan.decode_nb: the streaming kernel that cuts each expert's weights into whole-row slices */
@@ -76,8 +77,8 @@ typedef struct rd_plan {
                     this many columns (32, 64 or 128) of one expert; RD_DECODE_ROWS the one that gives it whole rows
                     for a slice of the contraction range (fp32 partial sums in the workspace, n <= 2048) or, with
                     trans_rhs, whole weight rows of a slice of the columns (no partial sums, k <= 8192) */
-  int split_k; /* rd_gmm only: 0 = when the tiles do not fill the device's last round and k >= 6400, cut those tiles'
-                  contraction range over up to sqrt(k)/20 work-groups (fp32 partial sums in the workspace); n > 0 =
+  int split_k; /* rd_gmm only: 0 = when the tiles do not fill the device's last round and k >= 6400 (float8: 12800), cut
+                  those tiles' contraction range over up to sqrt(k)/20 work-groups (fp32 partial sums in the workspace); n > 0 =
                   cut them over up to n (at most 8) whatever k is; -1 = never */
 } rd_plan;
 

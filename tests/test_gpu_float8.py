@@ -1,6 +1,7 @@
 """GPU parity for float8 e4m3fn operands (jax.lax.ragged_dot's float8 variant; the reference has no float8 path): the
-HIP kernels widen the bytes to bf16 on their way into LDS, multiply on the bf16 matrix cores with fp32 accumulation and
-store bf16.  Everything goes through the C ABI (ctypes).  The oracle decodes the bytes by the format's definition and
+HIP kernels multiply on the float8 matrix-core instruction where the row pitches are multiples of 16 bytes, and
+otherwise widen the bytes to bf16 on their way into LDS and multiply on the bf16 matrix cores; fp32 accumulation and
+bf16 output either way.  Everything goes through the C ABI (ctypes).  The oracle decodes the bytes by the format's definition and
 computes in float64; since products of two e4m3 values are exact in fp32, what is left is the fp32 accumulation order
 and the bf16 rounding of the result: the bf16 tolerances of the other parity tests apply unchanged."""
 
@@ -142,6 +143,48 @@ def test_float8_every_tile_shape(shape):
         assert not np.any(util.to_np(dA)[gs == 0])
         ran += 1
     assert ran >= 1
+
+
+@pytest.mark.parametrize("trans_rhs", [0, 1], ids=["nn", "nt"])
+@pytest.mark.parametrize("shape", [(900, 1104, 528, 5), (2100, 4112, 256, 3)], ids=lambda s: "m%d_k%d_n%d_g%d" % s)
+def test_float8_k_split_of_last_round(shape, trans_rhs):
+    """Few tiles and a long contraction on the float8 matrix-core shapes: the last round's tiles are cut along K over
+    several work-groups.  Matches the oracle, agrees with the unsplit run up to fp32 summation order, overwrites every
+    output element, and gives the same bits on a second call that reuses a workspace full of stale data."""
+    m, k, n, g = shape
+    x8, A8, _, gs, target_m = _case(11 + m, m, k, n, g)
+    gs[1] = 0
+    target_m = int(gs.sum())
+    xf, Af = oracle.float8_e4m3fn_to_f32(x8), oracle.float8_e4m3fn_to_f32(A8)
+    y_ref = oracle.gmm(xf, Af, gs)
+    x = _f8_dev(x8)
+    A = _f8_dev(np.ascontiguousarray(np.swapaxes(A8, 1, 2)) if trans_rhs else A8)
+    gs_d = torch.from_numpy(gs).cuda()
+    direct = [v for v in _f8_variants() if v.direct_to_lds]
+    assert direct
+    for v in direct:
+        print("float8 k-split", v.name.decode(), shape, "trans_rhs", trans_rhs, flush=True)
+        split, whole = _capi.Plan(v.id, 2, 0, 2, split_k=8), _capi.Plan(v.id, 2, 0, 2, split_k=-1)
+        need = _capi.lib.rd_gmm_workspace_bytes(m, g, ctypes.byref(split))
+        assert need > _capi.lib.rd_gmm_workspace_bytes(m, g, ctypes.byref(whole))
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        ws.fill_(0xA5)
+        outs = []
+        for plan in (split, split, whole):
+            y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+            rc = _capi.lib.rd_gmm(torch.cuda.current_stream().cuda_stream, x.data_ptr(), A.data_ptr(), gs_d.data_ptr(),
+                                  y.data_ptr(), m, k, n, g, trans_rhs, _capi.RD_DTYPE_F8E4M3_BF16, ctypes.byref(plan),
+                                  ws.data_ptr(), ws.numel())
+            torch.cuda.synchronize()
+            assert rc == 0, _capi.lib.rd_last_error()
+            outs.append(util.to_np(y))
+        for y in outs:
+            assert not np.isnan(y).any()
+            util.assert_close_rows(y, y_ref, target_m, util.BF16_EPS, "y")
+            assert not np.any(y[target_m:])
+        assert np.array_equal(outs[0], outs[1])
+        scale = np.abs(y_ref).max()
+        assert np.abs(outs[0].astype(np.float32) - outs[2].astype(np.float32)).max() <= 2 ** -7 * scale
 
 
 def test_float8_is_forward_only_and_rejects_mixed_operands():

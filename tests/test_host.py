@@ -100,7 +100,7 @@ def test_workspace_and_map_sizes():
             split = lib.rd_gmm_workspace_bytes(m, g, ctypes.byref(_capi.Plan(v.id)))
             extra = 256 * 4 + 256 * v.tile_m * v.tile_n * 4
             assert split in (whole, whole + extra), (v.name, split, whole)
-            if v.direct_to_lds and v.dtype == _capi.RD_DTYPE_BF16:  # (the float8 direct-to-LDS shapes have no K-split)
+            if v.direct_to_lds and v.dtype in (_capi.RD_DTYPE_BF16, _capi.RD_DTYPE_F8E4M3_BF16):
                 assert split == whole + extra and need >= split
 
 
