@@ -187,6 +187,40 @@ def test_float8_k_split_of_last_round(shape, trans_rhs):
         assert np.abs(outs[0].astype(np.float32) - outs[2].astype(np.float32)).max() <= 2 ** -7 * scale
 
 
+@pytest.mark.parametrize("trans_rhs", [0, 1], ids=["nn", "nt"])
+@pytest.mark.parametrize("k,split_k", [(80, -1), (1104, -1), (4112, 8), (2048, 3)], ids=["k80", "k1104", "k4112-split8", "k2048-split3"])
+def test_float8_short_group_row_tiles(k, split_k, trans_rhs):
+    """Groups of 1..64 rows (the 64-row streaming routine inside the 256 x 256 float8 kernel), longer ones and the short
+    last tile of a long group (tall routine) in one launch, contraction lengths that end inside a 128-deep and a 64-deep
+    slab, with and without the K-split; twice, same bits."""
+    vid = [v.id for v in _f8_variants() if v.direct_to_lds and v.tile_m == 256][0]
+    gs = np.array([5, 64, 65, 128, 129, 0, 33, 100, 1, 256, 300, 257, 640], np.int32)
+    m, n, g = int(gs.sum()) + 40, 528, gs.size
+    print(f"float8 short tiles k={k} split_k={split_k} trans_rhs={trans_rhs}", flush=True)
+    x8, A8, _, _, _ = _case(k, m, k, n, g, 1.0)
+    target_m = int(gs.sum())
+    y_ref = oracle.gmm(oracle.float8_e4m3fn_to_f32(x8), oracle.float8_e4m3fn_to_f32(A8), gs)
+    x = _f8_dev(x8)
+    A = _f8_dev(np.ascontiguousarray(np.swapaxes(A8, 1, 2)) if trans_rhs else A8)
+    gs_d = torch.from_numpy(gs).cuda()
+    plan = _capi.Plan(vid, 2, 0, 4, split_k=split_k)
+    ws = torch.empty(_capi.lib.rd_gmm_workspace_bytes(m, g, ctypes.byref(plan)), dtype=torch.uint8, device="cuda")
+    ws.fill_(0x3C)
+    prev = None
+    for _ in range(2):
+        y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        rc = _capi.lib.rd_gmm(torch.cuda.current_stream().cuda_stream, x.data_ptr(), A.data_ptr(), gs_d.data_ptr(),
+                              y.data_ptr(), m, k, n, g, trans_rhs, _capi.RD_DTYPE_F8E4M3_BF16, ctypes.byref(plan),
+                              ws.data_ptr(), ws.numel())
+        assert rc == 0, _capi.lib.rd_last_error()
+        torch.cuda.synchronize()
+        assert not torch.isnan(y).any()
+        util.assert_close_rows(util.to_np(y), y_ref, target_m, util.BF16_EPS, "y")
+        assert not torch.any(y[target_m:])
+        assert prev is None or torch.equal(prev, y)
+        prev = y
+
+
 def test_float8_is_forward_only_and_rejects_mixed_operands():
     x8, A8, _, gs, _ = _case(1, 128, 64, 64, 2)
     x, A = _f8_dev(x8), _f8_dev(A8)
