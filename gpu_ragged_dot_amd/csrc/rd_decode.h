@@ -26,7 +26,8 @@ int launch_gmm_rows(hipStream_t s, const DecodeArgs& a, int num_cus, void* works
 
 // The same for weights stored [g, n, k] (trans_rhs): the stream is cut along n, every piece yields complete sums, one
 // launch and no workspace.  DecodeArgs::A is then [g, n, k].  gmm_rows_t_fits: the shape can be served (k up to 8192).
-bool gmm_rows_t_fits(int m, int k, int n, int g);
-int launch_gmm_rows_t(hipStream_t s, const DecodeArgs& a, int num_cus);
+// f8: x and A hold float8 e4m3fn bytes behind the same pointers (k % 16 == 0); y is bf16 either way.
+bool gmm_rows_t_fits(int m, int k, int n, int g, bool f8 = false);
+int launch_gmm_rows_t(hipStream_t s, const DecodeArgs& a, int num_cus, bool f8 = false);
 
 }  // namespace rd

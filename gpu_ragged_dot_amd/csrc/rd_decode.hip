@@ -601,12 +601,19 @@ __device__ __forceinline__ float wave_sums(float (&v)[V], int lane) {
   return wave_sums_step<V, V, 32>(v, lane);
 }
 
-template <int RMAX>
+// F8: x and A hold float8 e4m3fn bytes (y is bf16 all the same).  A 16-byte chunk is then 16 contraction indices; the
+// activations are widened to bf16 as they are staged (two 16-byte entries per chunk, the chunk's lower and upper eight),
+// the weights as they are used (v_cvt_pk_f32_fp8 and a byte permute per pair, once per block of weight rows and shared
+// by the token rows), and the same v_dot2_f32_bf16 multiplies them - exactly, every e4m3 value being a bf16 value.
+template <int RMAX, bool F8>
 __global__ __launch_bounds__(kThreads, 2) void gmm_rows_t_kernel(DecodeArgs p, int wgs) {
+  constexpr int EB = F8 ? 1 : 2;     // bytes per element of x and A
+  constexpr int EPC = 16 / EB;       // elements per 16-byte chunk
+  constexpr int XE = F8 ? 2 : 1;     // staged 16-byte entries per chunk and token row
   __shared__ int32_t wave_cnt[2][kThreads / 64];
   __shared__ int32_t job[3];
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  u32x4_t* xs = reinterpret_cast<u32x4_t*>(smem_raw);  // [RMAX rows][chunk of 8 contraction indices] x 16 bytes
+  u32x4_t* xs = reinterpret_cast<u32x4_t*>(smem_raw);  // [RMAX rows][XE][chunk] x 16 bytes (8 bf16)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
   // which experts are non-empty and where their rows start (as in gmm_rows_kernel)
@@ -654,9 +661,10 @@ __global__ __launch_bounds__(kThreads, 2) void gmm_rows_t_kernel(DecodeArgs p, i
   if ((int)blockIdx.x >= experts_at_a_time * C) return;
   const int c = blockIdx.x % C;
   const int j_begin = c * per, j_end = imin(p.n, j_begin + per);
-  const int chunks = p.k >> 3;                        // 16-byte chunks per weight row (k % 8 == 0)
+  const int chunks = p.k / EPC;                       // 16-byte chunks per weight row (k % EPC == 0)
   const int npos = (chunks + 63) >> 6;                // loads per lane and weight row
-  const int r_stride = npos * 64;                     // staged entries per token row
+  const int r_stride = npos * 64;                     // staged chunks per token row
+  const unsigned char* xb = reinterpret_cast<const unsigned char*>(p.x);
 
   for (int want = blockIdx.x / C; want < n_act; want += experts_at_a_time) {
     __syncthreads();  // job free again
@@ -675,7 +683,7 @@ __global__ __launch_bounds__(kThreads, 2) void gmm_rows_t_kernel(DecodeArgs p, i
     const int gi = job[0], row0 = job[1];
     const int rows = imin(job[2], p.m - row0);
     if (rows <= 0) continue;
-    const bf16_bits* W = p.A + (size_t)gi * p.n * p.k;
+    const unsigned char* W = reinterpret_cast<const unsigned char*>(p.A) + (size_t)gi * p.n * p.k * EB;
     // this wave's weight rows: blocks of kTBlock consecutive rows, block wave, wave + 4, ... of the piece (a piece is a
     // whole number of blocks); its loads as one sequence of (block, position) steps of kTBlock loads each
     const int blocks = (j_end - j_begin) / kTBlock;
@@ -686,10 +694,11 @@ __global__ __launch_bounds__(kThreads, 2) void gmm_rows_t_kernel(DecodeArgs p, i
       const int sc = imin(s, nsteps - 1);
       const int i = sc / npos, q = sc - i * npos;
       const int ch = imin(q * 64 + lane, chunks - 1);
-      const uint32_t off = (uint32_t)(j_begin + kTBlock * (wave + 4 * i)) * (uint32_t)p.k + (uint32_t)ch * 8u;  // n * k < 2^31
+      // byte offsets: n * k < 2^31 elements
+      const uint32_t off = ((uint32_t)(j_begin + kTBlock * (wave + 4 * i)) * (uint32_t)p.k) * EB + (uint32_t)ch * 16u;
 #pragma unroll
       for (int b = 0; b < kTBlock; ++b)
-        dst[b] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(W + off + (uint32_t)b * (uint32_t)p.k));
+        dst[b] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(W + off + (uint32_t)b * (uint32_t)p.k * EB));
     };
 
     for (int rc = 0; rc < rows; rc += RMAX) {
@@ -700,22 +709,36 @@ __global__ __launch_bounds__(kThreads, 2) void gmm_rows_t_kernel(DecodeArgs p, i
         for (int u = 0; u < kTDepth; ++u) load_step(w[u], u);
       }
       __syncthreads();  // previous pass done with xs
-      // stage the activations: entry [row][chunk] = x[row][8 chunk .. 8 chunk + 7]; zero for rows past nr and for the
-      // chunks that pad the row to a whole number of positions (unconditional loads from clamped, valid addresses, four
-      // in flight per thread; masked afterwards)
+      // stage the activations: entry [row][chunk] = the chunk's 8 (float8: [row][0 / 1][chunk] = its lower / upper 8)
+      // contraction indices of x[row] as bf16; zero for rows past nr and for the chunks that pad the row to a whole
+      // number of positions (unconditional loads from clamped, valid addresses, four in flight per thread; masked
+      // afterwards)
       for (int base = 0; base < r_stride * RMAX; base += kThreads * 4) {
         u32x4_t v[4];
 #pragma unroll
         for (int s2 = 0; s2 < 4; ++s2) {
           const int idx = base + s2 * kThreads + tid;
           const int r = imin(idx / r_stride, nr - 1), ch = imin(idx % r_stride, chunks - 1);
-          v[s2] = *reinterpret_cast<const u32x4_t*>(p.x + (size_t)(row0 + rc + r) * p.k + (size_t)ch * 8);
+          v[s2] = *reinterpret_cast<const u32x4_t*>(xb + ((size_t)(row0 + rc + r) * p.k) * EB + (size_t)ch * 16);
         }
 #pragma unroll
         for (int s2 = 0; s2 < 4; ++s2) {
           const int idx = base + s2 * kThreads + tid;
-          const bool live = idx / r_stride < nr && idx % r_stride < chunks;
-          if (idx < r_stride * RMAX) xs[idx] = live ? v[s2] : u32x4_t{0, 0, 0, 0};
+          const int r = idx / r_stride, ch = idx - r * r_stride;
+          const bool live = r < nr && ch < chunks;
+          if (idx < r_stride * RMAX) {
+            if constexpr (F8) {
+              const uint32_t c0 = v[s2][0], c1 = v[s2][1], c2 = v[s2][2], c3 = v[s2][3];
+              const u32x4_t lo = {fp8e4m3x2_to_bf16x2<false>(c0), fp8e4m3x2_to_bf16x2<true>(c0),
+                                  fp8e4m3x2_to_bf16x2<false>(c1), fp8e4m3x2_to_bf16x2<true>(c1)};
+              const u32x4_t hi = {fp8e4m3x2_to_bf16x2<false>(c2), fp8e4m3x2_to_bf16x2<true>(c2),
+                                  fp8e4m3x2_to_bf16x2<false>(c3), fp8e4m3x2_to_bf16x2<true>(c3)};
+              xs[(2 * r) * r_stride + ch] = live ? lo : u32x4_t{0, 0, 0, 0};
+              xs[(2 * r + 1) * r_stride + ch] = live ? hi : u32x4_t{0, 0, 0, 0};
+            } else {
+              xs[idx] = live ? v[s2] : u32x4_t{0, 0, 0, 0};
+            }
+          }
         }
       }
       __syncthreads();
@@ -732,21 +755,37 @@ __global__ __launch_bounds__(kThreads, 2) void gmm_rows_t_kernel(DecodeArgs p, i
         for (int u = 0; u < kTDepth; ++u) {
           if (base + u < nsteps) {  // uniform over the wave
             const u32x4_t* xe = xs + (q * 64 + lane);
+            // the block's weights as pairs of bf16 (float8: widened here, once for all token rows).
+            // Scalars first: a bit cast applied to one element of a vector reads element 0 whatever the index.
+            uint32_t wp[kTBlock][4 * XE];
+#pragma unroll
+            for (int b = 0; b < kTBlock; ++b) {
+              const uint32_t w0 = w[u][b][0], w1 = w[u][b][1], w2 = w[u][b][2], w3 = w[u][b][3];
+              if constexpr (F8) {
+                wp[b][0] = fp8e4m3x2_to_bf16x2<false>(w0); wp[b][1] = fp8e4m3x2_to_bf16x2<true>(w0);
+                wp[b][2] = fp8e4m3x2_to_bf16x2<false>(w1); wp[b][3] = fp8e4m3x2_to_bf16x2<true>(w1);
+                wp[b][4] = fp8e4m3x2_to_bf16x2<false>(w2); wp[b][5] = fp8e4m3x2_to_bf16x2<true>(w2);
+                wp[b][6] = fp8e4m3x2_to_bf16x2<false>(w3); wp[b][7] = fp8e4m3x2_to_bf16x2<true>(w3);
+              } else {
+                wp[b][0] = w0; wp[b][1] = w1; wp[b][2] = w2; wp[b][3] = w3;
+              }
+            }
 #pragma unroll
             for (int r = 0; r < RMAX; ++r) {
-              // one read of the token row's 8 activations serves the block's kTBlock weight rows.
-              // Scalars first: a bit cast applied to one element of a vector reads element 0 whatever the index.
-              const u32x4_t xv = xe[(size_t)r * r_stride];
-              const uint32_t x0 = xv[0], x1 = xv[1], x2 = xv[2], x3 = xv[3];
+              // one read of the token row's activations serves the block's kTBlock weight rows
 #pragma unroll
-              for (int b = 0; b < kTBlock; ++b) {
-                const uint32_t w0 = w[u][b][0], w1 = w[u][b][1], w2 = w[u][b][2], w3 = w[u][b][3];
-                float a = acc[b][r];
-                a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w0), __builtin_bit_cast(bf16x2_t, x0), a, false);
-                a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w1), __builtin_bit_cast(bf16x2_t, x1), a, false);
-                a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w2), __builtin_bit_cast(bf16x2_t, x2), a, false);
-                a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w3), __builtin_bit_cast(bf16x2_t, x3), a, false);
-                acc[b][r] = a;
+              for (int h = 0; h < XE; ++h) {
+                const u32x4_t xv = xe[(size_t)(XE * r + h) * r_stride];
+                const uint32_t x0 = xv[0], x1 = xv[1], x2 = xv[2], x3 = xv[3];
+#pragma unroll
+                for (int b = 0; b < kTBlock; ++b) {
+                  float a = acc[b][r];
+                  a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, wp[b][4 * h + 0]), __builtin_bit_cast(bf16x2_t, x0), a, false);
+                  a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, wp[b][4 * h + 1]), __builtin_bit_cast(bf16x2_t, x1), a, false);
+                  a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, wp[b][4 * h + 2]), __builtin_bit_cast(bf16x2_t, x2), a, false);
+                  a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, wp[b][4 * h + 3]), __builtin_bit_cast(bf16x2_t, x3), a, false);
+                  acc[b][r] = a;
+                }
               }
             }
             if (++q == npos) {
@@ -870,25 +909,32 @@ int launch_gmm_rows(hipStream_t s, const DecodeArgs& a, int num_cus, void* works
   return (int)hipGetLastError();
 }
 
-// trans_rhs: A is [g, n, k].  Needs k % 8 == 0, n % 8 == 0, n * k < 2^31 and rows-per-pass x k (padded to 512) x 2
-// bytes of LDS within kTMaxLds.  No workspace.
-bool gmm_rows_t_fits(int m, int k, int n, int g) {
+// trans_rhs: A is [g, n, k].  Needs k % 8 == 0 (float8: 16), n % 8 == 0, n * k < 2^31 and rows-per-pass x k (padded to
+// 64 chunks of 16 bytes) x 2 bytes of LDS within kTMaxLds.  No workspace.
+bool gmm_rows_t_fits(int m, int k, int n, int g, bool f8) {
   (void)m; (void)n; (void)g;  // only the contraction length decides: 4 token rows of it must fit in LDS
-  const long long kpad = ((long long)k + 511) & ~511ll;
+  const long long pad = f8 ? 1023 : 511;
+  const long long kpad = ((long long)k + pad) & ~pad;
   return k > 0 && 4 * kpad * 2 <= kTMaxLds;
 }
 
-int launch_gmm_rows_t(hipStream_t s, const DecodeArgs& a, int num_cus) {
+int launch_gmm_rows_t(hipStream_t s, const DecodeArgs& a, int num_cus, bool f8) {
   if (a.m <= 0 || a.n <= 0 || a.g <= 0) return hipSuccess;
-  if (a.n % 8 != 0 || a.k % 8 != 0 || a.k <= 0) return hipErrorInvalidValue;
-  const int kpad = (a.k + 511) & ~511;
+  if (a.n % 8 != 0 || a.k % (f8 ? 16 : 8) != 0 || a.k <= 0) return hipErrorInvalidValue;
+  const int pad = f8 ? 1023 : 511;
+  const int kpad = (a.k + pad) & ~pad;
   const int wgs = 2 * (num_cus > 0 ? num_cus : 256);
   // more than one row per group on average and room for them: 8 token rows per pass over the weights, else 4
   const bool wide = a.m > a.g && (size_t)8 * kpad * 2 <= (size_t)kTMaxLds;
   const size_t lds = (size_t)(wide ? 8 : 4) * kpad * 2;
   if (lds > (size_t)kTMaxLds) return hipErrorInvalidValue;
-  if (wide) hipLaunchKernelGGL(gmm_rows_t_kernel<8>, dim3(wgs), dim3(kThreads), lds, s, a, wgs);
-  else hipLaunchKernelGGL(gmm_rows_t_kernel<4>, dim3(wgs), dim3(kThreads), lds, s, a, wgs);
+  if (f8) {
+    if (wide) hipLaunchKernelGGL((gmm_rows_t_kernel<8, true>), dim3(wgs), dim3(kThreads), lds, s, a, wgs);
+    else hipLaunchKernelGGL((gmm_rows_t_kernel<4, true>), dim3(wgs), dim3(kThreads), lds, s, a, wgs);
+  } else {
+    if (wide) hipLaunchKernelGGL((gmm_rows_t_kernel<8, false>), dim3(wgs), dim3(kThreads), lds, s, a, wgs);
+    else hipLaunchKernelGGL((gmm_rows_t_kernel<4, false>), dim3(wgs), dim3(kThreads), lds, s, a, wgs);
+  }
   return (int)hipGetLastError();
 }
 

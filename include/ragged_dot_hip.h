@@ -40,8 +40,9 @@ extern "C" {
  * accumulation); otherwise they are widened to bfloat16 as
  * they are loaded (exact: every e4m3 value is a bfloat16 value) and multiplied on the bf16 matrix cores.  Either way the
  * result is that of an exact-product fp32-accumulating float8 multiply; the first path has half the bytes to read and
- * twice the matrix-core rate of bfloat16, the second only the former.  Tile kernels only (no streaming kernel for a few
- * rows per group); the K-split of rd_plan.split_k on the first path only. */
+ * twice the matrix-core rate of bfloat16, the second only the former.  Of the streaming kernels for a few rows per group
+ * float8 has the one for weights stored [g, n, k] (trans_rhs, decode_nb = RD_DECODE_ROWS, k % 16 == 0; rd_default_plan
+ * picks it up to one row per group on average); the K-split of rd_plan.split_k on the first path only. */
 enum rd_dtype { RD_DTYPE_BF16 = 0, RD_DTYPE_F32 = 1, RD_DTYPE_F32_BF16 = 2, RD_DTYPE_F8E4M3_BF16 = 3 };
 
 #define RD_DECODE_ROWS (-1) /* rd_plan.decode_nb: the streaming kernel that cuts each expert's weights into whole-row slices */

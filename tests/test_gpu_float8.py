@@ -221,6 +221,77 @@ def test_float8_short_group_row_tiles(k, split_k, trans_rhs):
         prev = y
 
 
+F8_STREAM_CASES = {
+    "decode-shape": (2048, 768, None),
+    "long-groups-tail": (528, 200, np.array([0, 11, 1, 0, 9, 5], np.int32)),
+    "g600-sparse": (144, 72, None),
+    "g300-two-rows": (272, 40, None),
+    "wide-passes": (1040, 776, np.array([0, 1, 2, 3, 4, 5, 6, 7, 8, 0, 9, 12, 16, 17, 0, 3], np.int32)),
+    "k8192": (8192, 64, np.array([2, 0, 1, 3], np.int32)),
+    "n24": (2048, 24, np.array([1, 0, 4, 2, 0, 0, 1, 1], np.int32)),
+    "k16": (16, 136, np.array([3, 0, 1], np.int32)),
+}
+
+
+@pytest.mark.parametrize("case", list(F8_STREAM_CASES))
+def test_float8_streaming_kernel_trans_rhs(case):
+    """float8 weights stored [g, n, k] and a few rows per group: the streaming kernel that cuts every expert's weight
+    rows into blocks along n, widens the bytes to bf16 in registers and writes y in one launch.  By name and by the
+    default plan; 4 and 8 rows per pass, groups that need several passes, empty groups, a zero tail, contraction lengths
+    that are not a whole number of 1024-element positions, more non-empty groups than work-groups, fewer output columns
+    than pieces.  Its sums are those of the tile kernels up to fp32 addition order."""
+    print(f"float8 streaming kernel, trans_rhs, {case}", flush=True)
+    rng = np.random.default_rng(len(case))
+    k, n, gs = F8_STREAM_CASES[case]
+    if case == "decode-shape":
+        gs = np.zeros(128, np.int32)
+        np.add.at(gs, rng.integers(0, 128, 64), 1)
+    elif gs is None:
+        g, active, rows_each = (600, 40, 1) if case == "g600-sparse" else (300, 299, 2)
+        gs = np.zeros(g, np.int32)
+        gs[rng.choice(g, active, replace=False)] = rows_each
+    g, m = len(gs), int(gs.sum()) + 5
+    x8 = oracle.f32_to_float8_e4m3fn(rng.normal(size=(m, k)))
+    A8 = oracle.f32_to_float8_e4m3fn(rng.normal(size=(g, k, n)) / np.sqrt(k))
+    y_ref = oracle.gmm(oracle.float8_e4m3fn_to_f32(x8), oracle.float8_e4m3fn_to_f32(A8), gs)
+    At = _f8_dev(np.ascontiguousarray(np.swapaxes(A8, 1, 2)))
+    x, gs_t = _f8_dev(x8), torch.from_numpy(gs)
+    live = int(gs.sum())
+    if case == "decode-shape":
+        assert _capi.default_plan(_capi.OP_GMM_TRANS, m, k, n, g, _capi.RD_DTYPE_F8E4M3_BF16).decode_nb == _capi.RD_DECODE_ROWS
+    for plan in (_capi.Plan(-1, 0, _capi.RD_DECODE_ROWS), None):
+        y = util.to_np(ops._gmm_fwd(x, At, gs_t, **HP, trans_rhs=True, plan=plan))
+        util.assert_close_rows(y, y_ref, live, util.BF16_EPS, f"float8 trans_rhs streaming kernel plan={plan}")
+        assert not np.any(y[live:])
+    # forced onto a tile kernel: the same sums
+    tile = [v.id for v in _f8_variants() if not v.vec][0]
+    y_tile = util.to_np(ops._gmm_fwd(x, At, gs_t, **HP, trans_rhs=True, plan=_capi.Plan(tile)))
+    scale = max(np.abs(y_ref).max(), 1e-6)
+    assert np.abs(y.astype(np.float32) - y_tile.astype(np.float32)).max() <= 2 ** -6 * scale
+
+
+def test_float8_streaming_kernel_limits():
+    """What the float8 streaming kernel does not serve is refused by name and left to the tile kernels by default:
+    weights stored [g, k, n], a contraction too long to stage, a pitch that is not a multiple of 16."""
+    rng = np.random.default_rng(2)
+    gs = np.array([1, 2], np.int32)
+    for k, n, trans_rhs in ((512, 64, False), (8208, 16, True), (520, 64, True)):
+        x8 = oracle.f32_to_float8_e4m3fn(rng.normal(size=(3, k)))
+        A8 = oracle.f32_to_float8_e4m3fn(rng.normal(size=(2, k, n)) / np.sqrt(k))
+        y_ref = oracle.gmm(oracle.float8_e4m3fn_to_f32(x8), oracle.float8_e4m3fn_to_f32(A8), gs)
+        A = _f8_dev(np.ascontiguousarray(np.swapaxes(A8, 1, 2)) if trans_rhs else A8)
+        args = (_f8_dev(x8), A, torch.from_numpy(gs))
+        print(f"float8 streaming limits k={k} n={n} trans_rhs={trans_rhs}", flush=True)
+        for nb in (_capi.RD_DECODE_ROWS, 64):
+            if not trans_rhs:  # [g, k, n]: a streaming plan is dropped, as for every element type without those kernels
+                y = ops._gmm_fwd(*args, **HP, trans_rhs=False, plan=_capi.Plan(-1, 0, nb))
+                util.assert_close_rows(util.to_np(y), y_ref, 3, util.BF16_EPS, "dropped plan")
+                continue
+            with pytest.raises(_capi.RaggedDotError):
+                ops._gmm_fwd(*args, **HP, trans_rhs=trans_rhs, plan=_capi.Plan(-1, 0, nb))
+        util.assert_close_rows(util.to_np(ops._gmm_fwd(*args, **HP, trans_rhs=trans_rhs)), y_ref, 3, util.BF16_EPS, "default")
+
+
 def test_float8_is_forward_only_and_rejects_mixed_operands():
     x8, A8, _, gs, _ = _case(1, 128, 64, 64, 2)
     x, A = _f8_dev(x8), _f8_dev(A8)

@@ -131,6 +131,14 @@ def test_planner_choices():
     assert p.decode_nb == 0  # enough 256-column tiles for the tile kernels' streaming routines
     p = planner.select_plan(_capi.OP_GMM, 64, 7168, 2048, 256)
     assert p.decode_nb == _capi.RD_DECODE_ROWS
+    # float8: the streaming kernel for weights stored [g, n, k] only, up to one row per group on average
+    f8 = _capi.RD_DTYPE_F8E4M3_BF16
+    assert planner.select_plan(_capi.OP_GMM_TRANS, 64, 2048, 768, 128, dtype=f8).decode_nb == _capi.RD_DECODE_ROWS
+    assert planner.select_plan(_capi.OP_GMM_TRANS, 128, 2048, 768, 128, dtype=f8).decode_nb == _capi.RD_DECODE_ROWS
+    assert planner.select_plan(_capi.OP_GMM_TRANS, 256, 2048, 768, 128, dtype=f8).decode_nb == 0
+    assert planner.select_plan(_capi.OP_GMM_TRANS, 64, 2056, 768, 128, dtype=f8).decode_nb == 0  # k % 16
+    assert planner.select_plan(_capi.OP_GMM, 64, 2048, 768, 128, dtype=f8).decode_nb == 0
+    assert planner.select_plan(_capi.OP_GMM_TRANS, 64, 2048, 768, 128, dtype=_capi.RD_DTYPE_F32).decode_nb == 0
     p = planner.select_plan(_capi.OP_GMM, 16384, 4096, 14336, 8)
     assert vs[p.variant].tile_m == 256 and vs[p.variant].tile_n == 256
     p = planner.select_plan(_capi.OP_GMM, 16384, 4096, 14336, 8, block_m=128, block_k=64, block_n=128)
