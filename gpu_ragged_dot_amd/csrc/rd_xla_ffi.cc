@@ -26,6 +26,7 @@ namespace {
 int dtype_code(ffi::DataType t, bool compute_bf16) {
   if (t == ffi::DataType::BF16) return RD_DTYPE_BF16;
   if (t == ffi::DataType::F32) return compute_bf16 ? RD_DTYPE_F32_BF16 : RD_DTYPE_F32;
+  if (t == ffi::DataType::F8E4M3FN) return RD_DTYPE_F8E4M3_BF16;  // the result buffer is then bfloat16
   return -1;
 }
 
@@ -49,7 +50,7 @@ ffi::Error GmmImpl(hipStream_t stream, ffi::AnyBuffer x_buf, ffi::AnyBuffer A_bu
   if ((int)(trans_rhs ? A_buf.dimensions()[2] : A_buf.dimensions()[1]) != k || (int)gs_buf.dimensions()[0] != g)
     return ffi::Error(ffi::ErrorCode::kInvalidArgument, "rd_gmm: contraction or group count mismatch");
   const int dtype = dtype_code(x_buf.element_type(), compute_bf16);
-  if (dtype < 0) return ffi::Error(ffi::ErrorCode::kInvalidArgument, "rd_gmm: operands are bfloat16 or float32");
+  if (dtype < 0) return ffi::Error(ffi::ErrorCode::kInvalidArgument, "rd_gmm: operands are bfloat16, float32 or float8_e4m3fn");
   const rd_plan plan_value = {variant, group_m, group_n, decode_nb, split_k};
   const rd_plan* plan = &plan_value;
   const void* x = x_buf.untyped_data();
@@ -74,7 +75,7 @@ ffi::Error TgmmImpl(hipStream_t stream, ffi::AnyBuffer x_buf, ffi::AnyBuffer dy_
   const int m = (int)x_buf.dimensions()[0], k = (int)x_buf.dimensions()[1], n = (int)dy_buf.dimensions()[1];
   const int g = (int)gs_buf.dimensions()[0];
   const int dtype = dtype_code(x_buf.element_type(), compute_bf16);
-  if (dtype < 0) return ffi::Error(ffi::ErrorCode::kInvalidArgument, "rd_tgmm: operands are bfloat16 or float32");
+  if (dtype < 0) return ffi::Error(ffi::ErrorCode::kInvalidArgument, "rd_tgmm: operands are bfloat16, float32 or float8_e4m3fn");
   const rd_plan plan_value = {variant, group_m, group_n, decode_nb, split_k};
   const rd_plan* plan = &plan_value;
   const void* x = x_buf.untyped_data();

@@ -56,7 +56,14 @@ def _dtype_code(dtype, compute_dtype, acc_dtype) -> int:
         return _capi.RD_DTYPE_F32
     if dtype == jnp.float32 and compute == jnp.dtype(jnp.bfloat16):
         return _capi.RD_DTYPE_F32_BF16
+    if dtype == jnp.float8_e4m3fn and compute in (dtype, jnp.dtype(jnp.bfloat16), jnp.dtype(jnp.float32)):
+        return _capi.RD_DTYPE_F8E4M3_BF16  # jax.lax.ragged_dot with preferred_element_type=bfloat16; forward only
     raise NotImplementedError(f"no kernel for compute_dtype={compute_dtype} on {dtype} operands")
+
+
+def _out_dtype(dtype):
+    """The result has the operands' element type (gpu_ragged_dot.py:210,324); float8 operands give bfloat16."""
+    return jnp.bfloat16 if jnp.dtype(dtype) == jnp.float8_e4m3fn else dtype
 
 
 def _plan_attrs(plan: _capi.Plan) -> dict:
@@ -86,7 +93,7 @@ def _gmm_fwd(x, A, group_sizes, block_m, block_k, block_n, trans_rhs, interpret,
                                dtype=code)  # XLA buffers are at least 16-byte aligned
     ws_bytes = _capi.lib.rd_gmm_workspace_bytes(m, g, ctypes.byref(plan))
     with jax.named_scope("gpu_gmm"):  # :216
-        y, _ = jax.ffi.ffi_call("rd_gmm", (jax.ShapeDtypeStruct((m, n), x.dtype), _workspace(ws_bytes)))(
+        y, _ = jax.ffi.ffi_call("rd_gmm", (jax.ShapeDtypeStruct((m, n), _out_dtype(x.dtype)), _workspace(ws_bytes)))(
             x, A, group_sizes.astype(jnp.int32), trans_rhs=bool(trans_rhs), compute_bf16=code == _capi.RD_DTYPE_F32_BF16,
             chunk_m=np.int32(chunk_m), **_plan_attrs(plan))
     return y, (x, A, group_sizes)  # residuals, :227
@@ -106,7 +113,7 @@ def _tgmm_fwd(x, y, group_sizes, block_m, block_k, block_n, interpret, compute_d
     plan = planner.select_plan(_capi.OP_TGMM, m, k, n, g, block_m, block_k, block_n, dtype=code)
     ws_bytes = _capi.lib.rd_tgmm_workspace_bytes(m, g, ctypes.byref(plan))
     with jax.named_scope("gpu_tgmm"):  # :330
-        out, _ = jax.ffi.ffi_call("rd_tgmm", (jax.ShapeDtypeStruct((g, k, n), x.dtype), _workspace(ws_bytes)))(
+        out, _ = jax.ffi.ffi_call("rd_tgmm", (jax.ShapeDtypeStruct((g, k, n), _out_dtype(x.dtype)), _workspace(ws_bytes)))(
             x, y, group_sizes.astype(jnp.int32), compute_bf16=code == _capi.RD_DTYPE_F32_BF16, chunk_m=np.int32(chunk_m),
             **_plan_attrs(plan))
     return out, (x, y, group_sizes)
