@@ -2,7 +2,7 @@
 
 Called through the C ABI and compared with rd_gmm on the same inputs and plan: same kernels, so bit-exact.  Two calls
 in a row, the second on a smaller input, for the tile kernels and for the streaming (few rows per group) kernels, and
-again on float32 arrays; sizes beyond the scratch buffer are refused with RD_ERR_WORKSPACE.
+again on float32 and float8 arrays; sizes beyond the scratch buffer are refused with RD_ERR_WORKSPACE.
 """
 
 import ctypes
@@ -79,6 +79,31 @@ def test_noalloc_float32_arrays():
             x, A, gs_d = torch.from_numpy(lhs).cuda(), torch.from_numpy(rhs).cuda(), torch.from_numpy(gs).cuda()
             ref, got = _run_both(x, A, gs_d, m, k, n, g, False, dtype, None, torch.float32)
             assert torch.equal(got, ref)
+
+
+def test_noalloc_float8_operands():
+    """float8 e4m3fn operands (bf16 out): the float8 matrix-core tiles in both weight layouts, and the streaming kernel
+    for weights stored [g, n, k] (the default plan's choice for one row per group)."""
+    for m, k, n, g, trans_rhs, streaming in ((600, 272, 528, 5, False, False), (300, 144, 272, 3, True, False),
+                                             (40, 528, 264, 48, True, True), (12, 144, 72, 20, True, True)):
+        print(f"noalloc float8 m={m} k={k} n={n} g={g} trans_rhs={trans_rhs}", flush=True)
+        rng = np.random.default_rng(m)
+        x8 = oracle.f32_to_float8_e4m3fn(rng.normal(size=(m, k)))
+        A8 = oracle.f32_to_float8_e4m3fn(rng.normal(size=(g, k, n)) / np.sqrt(k))
+        if streaming:
+            gs = np.zeros(g, np.int32)
+            gs[rng.choice(g, m - 3, replace=False)] = 1
+            assert _capi.default_plan(_capi.OP_GMM_TRANS, m, k, n, g, _capi.RD_DTYPE_F8E4M3_BF16).decode_nb == _capi.RD_DECODE_ROWS
+        else:
+            gs = oracle.generate_group_sizes(m, g, m - 11)
+        live = int(gs.sum())
+        x = torch.from_numpy(x8).cuda().view(torch.float8_e4m3fn)
+        A = torch.from_numpy(np.ascontiguousarray(np.swapaxes(A8, 1, 2)) if trans_rhs else A8).cuda().view(torch.float8_e4m3fn)
+        ref, got = _run_both(x, A, torch.from_numpy(gs).cuda(), m, k, n, g, trans_rhs, _capi.RD_DTYPE_F8E4M3_BF16, None, torch.bfloat16)
+        assert torch.equal(got, ref)
+        y_ref = oracle.gmm(oracle.float8_e4m3fn_to_f32(x8), oracle.float8_e4m3fn_to_f32(A8), gs)
+        util.assert_close_rows(util.to_np(got), y_ref, live, util.BF16_EPS, "y")
+        assert not np.any(util.to_np(got)[live:])
 
 
 def test_noalloc_refuses_what_does_not_fit():
