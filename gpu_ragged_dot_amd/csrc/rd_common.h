@@ -29,14 +29,14 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 typedef uint8_t fp8_bits;  // storage type of an OCP float8 e4m3fn element in HBM
 
 // float8 e4m3fn (1 sign, 4 exponent bits of bias 7, 3 mantissa bits; no infinities, S.1111.111 is NaN) -> bf16.  Every
-// e4m3 value is a bf16 value, so this is exact: the hardware widens to fp32 (gfx950's float8 is this format) and the
-// upper half of the fp32 word is the bf16.
-// The two float8 bytes of the lower (HI = false) or upper half of w, as a pair of bf16.
+// e4m3 value is a bf16 value, so this is exact (gfx950's float8 is this format).
+// The two float8 bytes of the lower (HI = false) or upper half of w, as a pair of bf16: v_cvt_scalef32_pk_bf16_fp8 with
+// a scale of one (checked on all 65536 pairs of codes against v_cvt_pk_f32_fp8 and the upper halves of its fp32 words).
 template <bool HI>
 __device__ __forceinline__ uint32_t fp8e4m3x2_to_bf16x2(uint32_t w) {
-  const f32x2_t f = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, HI);
-  // bytes 2-3 of each fp32 word: [f[1].b3 f[1].b2 f[0].b3 f[0].b2]
-  return __builtin_amdgcn_perm(__float_as_uint(f[1]), __float_as_uint(f[0]), 0x07060302u);
+  typedef __bf16 bf16x2_raw_t __attribute__((ext_vector_type(2)));
+  const bf16x2_raw_t v = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, HI);
+  return __builtin_bit_cast(uint32_t, v);
 }
 __device__ __forceinline__ uint32_t fp8e4m3_to_bf16(uint32_t b) {
   return fp8e4m3x2_to_bf16x2<false>(b & 0xff) & 0xffff;

@@ -603,7 +603,7 @@ __device__ __forceinline__ float wave_sums(float (&v)[V], int lane) {
 
 // F8: x and A hold float8 e4m3fn bytes (y is bf16 all the same).  A 16-byte chunk is then 16 contraction indices; the
 // activations are widened to bf16 as they are staged (two 16-byte entries per chunk, the chunk's lower and upper eight),
-// the weights as they are used (v_cvt_pk_f32_fp8 and a byte permute per pair, once per block of weight rows and shared
+// the weights as they are used (one v_cvt_scalef32_pk_bf16_fp8 per pair, once per block of weight rows and shared
 // by the token rows), and the same v_dot2_f32_bf16 multiplies them - exactly, every e4m3 value being a bf16 value.
 template <int RMAX, bool F8>
 __global__ __launch_bounds__(kThreads, 2) void gmm_rows_t_kernel(DecodeArgs p, int wgs) {
