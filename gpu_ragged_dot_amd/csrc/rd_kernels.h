@@ -255,14 +255,16 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
       }
     }
     if constexpr (IsF8Direct<C>::value) {
-      if constexpr (C::PINGPONG && C::A_KMAJOR && C::BM > kShortRows) {
+      if constexpr (C::NW == 8 && C::WAVES_M == 2 && C::A_KMAJOR && C::BM > kShortRows) {
         // a group's single row tile of at most kShortRows rows, as above: a 64-row routine on 128-deep slabs (every load
-        // covers whole 128-byte lines), the weights streamed past L2
-        if (rows <= kShortRows && it == 0) {
-          typedef F8Cfg<kShortRows, C::BN, 2, 4, 3, 128, kCachePolicyStream, true, C::B_KMAJOR, false> S;
-          static_assert(S::LDS_BYTES <= C::LDS_BYTES && S::NT == C::NT, "the short routine runs in the tall one's launch");
-          gemm_tile_f8<S>(Ap, p.k, rows, Bp, TRANS_RHS ? p.k : p.n, cols, klen, Op, p.n, smem, sk);
-          return;
+        // covers whole 128-byte lines), the weights streamed past L2 - where the tall routine's LDS has room for its ring
+        typedef F8Cfg<kShortRows, C::BN, 2, 4, 3, 128, kCachePolicyStream, true, C::B_KMAJOR, false> S;
+        if constexpr (S::LDS_BYTES <= C::LDS_BYTES) {
+          static_assert(S::NT == C::NT, "the short routine runs in the tall one's launch");
+          if (rows <= kShortRows && it == 0) {
+            gemm_tile_f8<S>(Ap, p.k, rows, Bp, TRANS_RHS ? p.k : p.n, cols, klen, Op, p.n, smem, sk);
+            return;
+          }
         }
       }
     }
