@@ -30,6 +30,13 @@ int dtype_code(ffi::DataType t, bool compute_bf16) {
   return -1;
 }
 
+// Element type of the product for operands of type t: their own, except that float8 operands give bfloat16 (the
+// Python side declares the result that way, jax_adapter._out_dtype).
+ffi::DataType result_type(ffi::DataType t) {
+  if (t == ffi::DataType::F8E4M3FN) return ffi::DataType::BF16;
+  return t;
+}
+
 ffi::Error status(int rc) {
   if (rc == RD_OK) return ffi::Error::Success();
   return ffi::Error(rc == RD_ERR_HIP ? ffi::ErrorCode::kInternal : ffi::ErrorCode::kInvalidArgument, rd_last_error());
@@ -41,8 +48,9 @@ ffi::Error GmmImpl(hipStream_t stream, ffi::AnyBuffer x_buf, ffi::AnyBuffer A_bu
                    int32_t split_k, int32_t chunk_m) {
   if (x_buf.dimensions().size() != 2 || A_buf.dimensions().size() != 3 || gs_buf.dimensions().size() != 1)
     return ffi::Error(ffi::ErrorCode::kInvalidArgument, "rd_gmm: x is [m,k], A is [g,k,n] or [g,n,k], group_sizes is [g]");
-  if (A_buf.element_type() != x_buf.element_type() || y_buf->element_type() != x_buf.element_type())
-    return ffi::Error(ffi::ErrorCode::kInvalidArgument, "rd_gmm: x, A and y must have one element type");
+  if (A_buf.element_type() != x_buf.element_type() || y_buf->element_type() != result_type(x_buf.element_type()))
+    return ffi::Error(ffi::ErrorCode::kInvalidArgument,
+                      "rd_gmm: x and A must have one element type and y that of the product (bfloat16 for float8 operands)");
   if (chunk_m < 1) return ffi::Error(ffi::ErrorCode::kInvalidArgument, "rd_gmm: chunk_m must be positive");
   const int trans_rhs = trans_rhs_attr ? 1 : 0;
   const int m = (int)x_buf.dimensions()[0], k = (int)x_buf.dimensions()[1], g = (int)A_buf.dimensions()[0];
@@ -69,8 +77,9 @@ ffi::Error TgmmImpl(hipStream_t stream, ffi::AnyBuffer x_buf, ffi::AnyBuffer dy_
   if (x_buf.dimensions().size() != 2 || dy_buf.dimensions().size() != 2 || gs_buf.dimensions().size() != 1 ||
       x_buf.dimensions()[0] != dy_buf.dimensions()[0])  // gpu_ragged_dot.py:304
     return ffi::Error(ffi::ErrorCode::kInvalidArgument, "rd_tgmm: x is [m,k], y is [m,n], group_sizes is [g]");
-  if (dy_buf.element_type() != x_buf.element_type() || dA_buf->element_type() != x_buf.element_type())
-    return ffi::Error(ffi::ErrorCode::kInvalidArgument, "rd_tgmm: x, y and the result must have one element type");
+  if (dy_buf.element_type() != x_buf.element_type() || dA_buf->element_type() != result_type(x_buf.element_type()))
+    return ffi::Error(ffi::ErrorCode::kInvalidArgument,
+                      "rd_tgmm: x and y must have one element type and the result that of the product (bfloat16 for float8 operands)");
   (void)chunk_m;  // accepted and unused, as gpu_ragged_dot.py:303
   const int m = (int)x_buf.dimensions()[0], k = (int)x_buf.dimensions()[1], n = (int)dy_buf.dimensions()[1];
   const int g = (int)gs_buf.dimensions()[0];

@@ -117,3 +117,48 @@ def test_handlers_pass_arguments_in_header_order():
         assert bound == want, (symbol, bound)
     # element type comes from the buffer, never hard-coded
     assert "element_type()" in shim and not re.search(r"rd_t?gmm\([^;]*RD_DTYPE_BF16", shim)
+
+
+def _shim_function(shim, name):
+    """Body of a free function of the shim, braces balanced."""
+    start = re.search(r"\b" + name + r"\s*\([^)]*\)\s*\{", shim)
+    assert start, name
+    depth, i = 1, start.end()
+    while depth:
+        depth += {"{": 1, "}": -1}.get(shim[i], 0)
+        i += 1
+    return shim[start.end():i - 1]
+
+
+def test_result_element_type_rule_matches_the_python_side():
+    """The handlers must accept exactly the result buffer jax_adapter declares (gpu_ragged_dot.py:210,324: the operands'
+    type; float8 operands give bfloat16).  The shim's rule is evaluated from its source for every element type
+    dtype_code() knows and compared with jax_adapter._out_dtype evaluated from its source."""
+    with open(SHIM) as f:
+        shim = f.read()
+    # element types the shim accepts
+    known = re.findall(r"t == ffi::DataType::([A-Z0-9]+)", _shim_function(shim, "dtype_code"))
+    assert sorted(known) == ["BF16", "F32", "F8E4M3FN"], known
+    # result_type(): `if (t == ffi::DataType::X) return ffi::DataType::Y;` lines, then `return t;`
+    body = _shim_function(shim, "result_type")
+    special = dict(re.findall(r"if \(t == ffi::DataType::([A-Z0-9]+)\) return ffi::DataType::([A-Z0-9]+);", body))
+    assert re.search(r"return t;\s*$", body.strip())
+    shim_rule = {t: special.get(t, t) for t in known}
+    # jax_adapter._out_dtype evaluated with stand-ins for jnp
+    names = {"BF16": "bfloat16", "F32": "float32", "F8E4M3FN": "float8_e4m3fn"}
+
+    class _Jnp:
+        bfloat16, float32, float8_e4m3fn = "bfloat16", "float32", "float8_e4m3fn"
+        dtype = staticmethod(lambda d: d)
+
+    fn = _func(_tree(), "_out_dtype")
+    scope = {"jnp": _Jnp}
+    exec(compile(ast.Module(body=[fn], type_ignores=[]), ADAPTER, "exec"), scope)
+    for t in known:
+        assert names[shim_rule[t]] == scope["_out_dtype"](names[t]), (t, shim_rule[t])
+    # both handlers check the result against that rule, and the operands against each other
+    for impl, res, other in (("GmmImpl", "y_buf", "A_buf"), ("TgmmImpl", "dA_buf", "dy_buf")):
+        body = _shim_function(shim, impl)
+        assert f"{res}->element_type() != result_type(x_buf.element_type())" in body, impl
+        assert f"{other}.element_type() != x_buf.element_type()" in body, impl
+        assert f"{res}->element_type() != x_buf.element_type()" not in body, impl
