@@ -7,8 +7,8 @@ workloads, forward + dlhs + drhs for the others.  Prints ONE JSON line.  Its top
 workload (default: the Mixtral-8x7B-shaped forward+backward).  Unless --only is given, the same line also carries
   "configs": the other measured configurations (mixtral_fwd, deepseek_fwd_bwd, decode), each with ms_per_step, value,
              roofline and cpu_baseline of its own;
-  "context": what the same box does with a dense bf16 GEMM of the Mixtral forward's size (torch.matmul, on N(0,1)
-             data and on zeros), a sustained (>= 2 s) loop of the headline step, a bare read of the decode shape's
+  "context": what the same box does with a dense bf16 GEMM of the Mixtral forward's size (torch.matmul and this
+             library's own kernels with one group, on N(0,1) data and on zeros), a sustained (>= 2 s) loop of the headline step, a bare read of the decode shape's
              bytes, the decode shape with its weights stored [g, n, k] (trans_rhs), the Mixtral-shaped products on float8
              operands, and the CPU model.
 """
@@ -285,10 +285,12 @@ def dense_gemm_context(torch):
     """hipBLASLt (torch.matmul) on dense bf16 GEMMs with the FLOPs of one Mixtral product, on N(0,1) data and on zeros:
     what the vendor library reaches on this box, and how much the data (power) matters.  Three operand layouts, those
     of the three products: forward x[m,k].W[k,n]; dlhs dout[m,n].W[k,n]^T (both operands run along the contraction
-    index); drhs x[m,k]^T.dout[m,n]."""
+    index); drhs x[m,k]^T.dout[m,n].  Returns that and, second, this library's own kernels on the same operands."""
+    from gpu_ragged_dot_amd import ops
+
     m, k, n = 16384, 4096, 14336
     gen = torch.Generator(device="cuda").manual_seed(7)
-    out = {}
+    out, own = {}, {}
     for label in ("normal", "zeros"):
         if label == "normal":
             a = torch.randn((m, k), generator=gen, device="cuda").to(torch.bfloat16)
@@ -308,8 +310,24 @@ def dense_gemm_context(torch):
                 fn()
             ms = _event_ms(fn, 30, torch)
             out[label + suffix] = {"ms": ms, "TFLOP/s": 2.0 * m * k * n / (ms * 1e-3) / 1e12}
+        # this library's kernels on the very same operands as ONE group of m rows (a dense GEMM through the product
+        # code, default plans): the gap to the vendor kernel per layout, and zeros against N(0,1) (the power limit)
+        one = torch.tensor([m], dtype=torch.int32, device="cuda")
+        b3 = b.unsqueeze(0)
+        hp = dict(HP, acc_dtype=torch.float32)
+        own_layouts = (("", lambda: ops._gmm_fwd(a, b3, one, **hp, trans_rhs=False)),
+                       ("_dlhs_layout", lambda: ops._gmm_fwd(d, b3, one, **hp, trans_rhs=True)),
+                       ("_drhs_layout", lambda: ops._tgmm_fwd(a, d, one, **hp)))
+        for suffix, fn in own_layouts:
+            for _ in range(3):
+                fn()
+            ms = _event_ms(fn, 20, torch)
+            own[label + suffix] = {"ms": ms, "TFLOP/s": 2.0 * m * k * n / (ms * 1e-3) / 1e12}
+        del a, b, d, c, ca, cb, b3
+    own["what"] = ("this library (ops._gmm_fwd / _tgmm_fwd, default plans) on the same operands as one group of 16384 "
+                   "rows: forward, trans_rhs (dlhs layout), tgmm (drhs layout)")
     return {"what": "torch.matmul bf16, m16384 k4096 n14336: x.W (the Mixtral forward's FLOPs as one dense GEMM), "
-                    "dout.W^T (dlhs layout), x^T.dout (drhs layout)", **out}
+                    "dout.W^T (dlhs layout), x^T.dout (drhs layout)", **out}, own
 
 
 def float8_context(torch):
@@ -468,7 +486,8 @@ def main():
                 c["cpu_baseline"] = cpu_baseline(other, args.cpu_seconds)
             configs[other] = c
         out["configs"] = configs
-        out["context"] = {"dense_gemm": dense_gemm_context(torch), "sustained_headline_step": out.pop("sustained", None),
+        vendor_dense, own_dense = dense_gemm_context(torch)
+        out["context"] = {"dense_gemm": vendor_dense, "own_dense_gemm": own_dense, "sustained_headline_step": out.pop("sustained", None),
                           "decode_bare_stream": configs["decode"].pop("bare_stream", None),
                           "decode_trans_rhs": configs["decode"].pop("trans_rhs", None),
                           "float8_mixtral_products": float8_context(torch), "cpu": cpu_model(),

@@ -160,7 +160,8 @@ int rd_tgmm(void* stream, const void* x, const void* dy, const int32_t* group_si
             size_t workspace_bytes);
 
 /* ---- measurement aid ----------------------------------------------------------------------------------------------
- * No counterpart in the reference.  A load-only kernel: reads `bytes` (src 16-byte aligned) cut into contiguous blocks
+ * No counterpart in the reference and not part of the surface that replaces it: nothing a caller of ragged_dot needs,
+ * only what the benchmark uses to time a bare read on the same device in the same process.  A load-only kernel: reads `bytes` (src 16-byte aligned) cut into contiguous blocks
  * of block_bytes, one work-group per block, and stores nothing (`sink`, 4 bytes of device memory or NULL, is written
  * only if the folded data equals one fixed word).  It is what a bare stream over the same bytes takes on this device -
  * the floor the benchmark prints next to the memory-bound kernels. */

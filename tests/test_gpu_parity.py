@@ -146,6 +146,42 @@ def test_every_variant(vid, vname, vec, shape):
     assert not np.any(util.to_np(dA)[gs == 0])
 
 
+def _tall_tgmm_variants():
+    return [(v.id, v.name.decode()) for v in _capi.variants()
+            if v.dtype == _capi.RD_DTYPE_BF16 and v.direct_to_lds and v.tile_m == 256 and v.tile_n == 256]
+
+
+@pytest.mark.parametrize("vid,vname", _tall_tgmm_variants(), ids=[v[1] for v in _tall_tgmm_variants()])
+@pytest.mark.parametrize("group_m", [1, 4])
+def test_tgmm_group_length_classes(vid, vname, group_m):
+    """tgmm of the 256 x 256 cores on a launch with several tiles per compute unit and groups of every length class -
+    empty, one slab of the K loop, two, three (the prologue's depth), more, a long one, next to each other in every
+    order - with ragged edges in k and n, a zero tail, and a second call on other data."""
+    from gpu_ragged_dot_amd import ops
+    print(f"tgmm length classes {vname} group_m={group_m}", flush=True)
+    k, n = 1288, 1544            # 6 x 7 tiles per group, the last ones partial
+    lens = [0, 1, 31, 32, 33, 64, 65, 96, 97, 127, 128, 129, 160, 300, 0, 0, 7, 1100, 5, 0, 40, 200, 95, 2, 0, 64, 31, 513, 96, 33]
+    rng = np.random.default_rng(11)
+    gs = np.array(lens, np.int32)
+    g = len(lens)
+    assert g * 6 * 7 >= 4 * 256   # several tiles per compute unit
+    m = int(gs.sum()) + 37
+    hp = dict(block_m=64, block_k=64, block_n=64, interpret=False, compute_dtype=None, acc_dtype=torch.float32, chunk_m=512)
+    plan = _capi.Plan(vid, group_m, 0)
+    for scale in (1.0, -2.0):
+        lhs = oracle.round_to(scale * rng.standard_normal((m, k)).astype(np.float32), "bfloat16")
+        dout = oracle.round_to(rng.standard_normal((m, n)).astype(np.float32), "bfloat16")
+        out = util.to_np(ops._tgmm_fwd(util.bf16_dev(lhs), util.bf16_dev(dout), torch.from_numpy(gs), **hp, plan=plan))
+        ref = oracle.tgmm(lhs, dout, gs)
+        util.assert_close_groups(out, ref, gs != 0, util.TGMM_BF16_EPS, f"tgmm scale={scale}")
+        assert not np.any(out[gs == 0])
+    # all-ones operands give every element its group's row count, exactly
+    ones_x, ones_d = np.ones((m, k), np.float32), np.ones((m, n), np.float32)
+    out = util.to_np(ops._tgmm_fwd(util.bf16_dev(ones_x), util.bf16_dev(ones_d), torch.from_numpy(gs), **hp, plan=plan))
+    want = oracle.round_to(gs.astype(np.float32), "bfloat16")[:, None, None] * np.ones((1, k, n), np.float32)
+    assert np.array_equal(out, want)
+
+
 def _split_variants():
     return [(v.id, v.name.decode()) for v in _capi.variants() if v.dtype == _capi.RD_DTYPE_BF16 and v.direct_to_lds]
 
@@ -518,6 +554,47 @@ def test_float32_every_tile_shape(shape):
         assert float(np.max(oracle.err_fn(util.to_np(dr), drhs_ref, axis=(-1, -2), mask=gs != 0))) < F32_TGMM_EPS
         assert not np.any(util.to_np(o)[m - 37:]) and not np.any(util.to_np(dl)[m - 37:])
         assert not np.any(util.to_np(dr)[gs == 0])
+
+
+def test_streaming_default_with_all_rows_in_one_group():
+    """The shape-only default picks the streaming kernel for m <= 4 g; the shape cannot see that all rows sit in one
+    group, whose weights are then streamed once per 8 rows.  Slow (the header says so) but it must be right."""
+    print("streaming default, all rows in one group", flush=True)
+    m, k, n, g = 256, 2048, 768, 128
+    assert _capi.default_plan(_capi.OP_GMM, m, k, n, g).decode_nb == _capi.RD_DECODE_ROWS
+    rng = np.random.default_rng(77)
+    lhs = oracle.round_to(rng.standard_normal((m, k)).astype(np.float32), "bfloat16")
+    rhs = oracle.round_to((rng.standard_normal((g, k, n)) / k ** 0.5).astype(np.float32), "bfloat16")
+    for hot in (0, 77, g - 1):
+        gs = np.zeros(g, np.int32)
+        gs[hot] = m
+        x, A, gsd = util.bf16_dev(lhs), util.bf16_dev(rhs), torch.from_numpy(gs).cuda()
+        for trans_rhs in (False, True):
+            Ad = A.mT.contiguous() if trans_rhs else A
+            y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+            assert _raw_gmm(x, Ad, gsd, y, trans_rhs=trans_rhs) == _capi.RD_OK, _capi.lib.rd_last_error()
+            util.assert_close_rows(util.to_np(y), oracle.gmm(lhs, rhs, gs), m, util.BF16_EPS, f"hot={hot} t={trans_rhs}")
+
+
+def test_stream_read_probe():
+    """rd_probe_stream_read is a measurement aid, not part of the drop-in surface: it must run, store nothing, and
+    refuse a source that is not 16-byte aligned."""
+    print("stream read probe", flush=True)
+    src = torch.arange(1 << 20, dtype=torch.int32, device="cuda")
+    sink = torch.full((1,), 0x5a5a5a5a, dtype=torch.int32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    for block in (16, 4096, 64 << 10, 3 << 20, 16 << 20):   # one thread's load .. more than the buffer
+        rc = _capi.lib.rd_probe_stream_read(stream, src.data_ptr(), src.numel() * 4, block, sink.data_ptr())
+        assert rc == _capi.RD_OK, _capi.lib.rd_last_error()
+    assert _capi.lib.rd_probe_stream_read(stream, src.data_ptr(), src.numel() * 4 - 12, 4096, None) == _capi.RD_OK
+    assert _capi.lib.rd_probe_stream_read(stream, src.data_ptr(), 0, 4096, None) == _capi.RD_OK
+    torch.cuda.synchronize()
+    assert int(sink.item()) == 0x5a5a5a5a
+    assert torch.equal(src, torch.arange(1 << 20, dtype=torch.int32, device="cuda"))
+    rc = _capi.lib.rd_probe_stream_read(stream, src.data_ptr() + 4, 4096, 4096, None)
+    assert rc == _capi.RD_ERR_INVALID_ARGUMENT
+    assert _capi.lib.rd_probe_stream_read(stream, src.data_ptr(), 4096, 8, None) == _capi.RD_ERR_INVALID_ARGUMENT
+    assert _capi.lib.rd_probe_stream_read(stream, None, 4096, 4096, None) == _capi.RD_ERR_INVALID_ARGUMENT
 
 
 # ---------------------------------------------------------------------------------------------------------------------
