@@ -419,61 +419,89 @@ __device__ __forceinline__ void wide_pass(const DecodeArgs& p, int rps, int unit
 template <bool WIDE>
 __global__ __launch_bounds__(kThreads, 2) void gmm_rows_kernel(DecodeArgs p, RowsGeom q, RowsHeader* __restrict__ header,
                                                                float* __restrict__ partials) {
-  __shared__ int32_t wave_cnt[2][kThreads / 64];
-  __shared__ int32_t job[3];                // expert, first row, rows of the expert this work-group serves
+  __shared__ int32_t wave_cnt[3][kThreads / 64];
+  __shared__ int32_t job[3];                // expert, first row and row count of the pass this work-group serves
+  constexpr int RPP = WIDE ? kWideRows : kRows;  // rows per pass
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   u32x2_t* xs = reinterpret_cast<u32x2_t*>(smem_raw);                   // [kMaxSeg] x {4 rows as bf16}
   float* part = reinterpret_cast<float*>(smem_raw + (WIDE ? kXsBytes : kMaxSeg * 8));  // [rps][rows per pass][n]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
   // ---- which experts are non-empty, and where their rows start: a scan over the group sizes --------------------------
-  // One slab of kThreads experts at a time: every thread learns how many non-empty experts and rows precede its own.
-  // With g <= kThreads (the usual case) the group sizes are read once and the result stays in registers.
+  // One slab of kThreads experts at a time: every thread learns how many jobs and rows precede its own expert's.  A job
+  // is one pass over an expert's weights with up to RPP of its rows: an expert with more rows than a pass holds is
+  // several jobs, served by different work-groups at the same time - if all rows of a call pile up in one group, its
+  // weights are streamed by all work-groups together (out of L2 after the first pass) instead of pass after pass by a
+  // few.  With g <= kThreads (the usual case) the group sizes are read once and the result stays in registers.
   auto scan_slab = [&](int base, int seen, int rows_seen, int& sz, int& rank, int& first_row, int& slab_act, int& slab_rows) {
     const int e = base + tid;
-    sz = e < p.g ? imax(p.group_sizes[e], 0) : 0;
+    sz = e < p.g ? imin(imax(p.group_sizes[e], 0), p.m) : 0;  // (no group has more than m rows that exist)
+    const int units = (sz + RPP - 1) / RPP;  // passes over this expert's weights, each a job of its own
     const unsigned long long m_act = __ballot(sz > 0);
-    const int before_in_wave = __popcll(m_act & ((1ull << lane) - 1ull));
+    const bool wave_big = __ballot(sz > RPP) != 0;  // some expert of this wave takes more than one pass
     int incl = sz;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) { const int up = __shfl_up(incl, d, 64); if (lane >= d) incl += up; }
     __syncthreads();  // wave_cnt free again
-    if (lane == 63) { wave_cnt[0][wave] = __popcll(m_act); wave_cnt[1][wave] = incl; }
+    if (lane == 63) { wave_cnt[0][wave] = __popcll(m_act); wave_cnt[1][wave] = incl; wave_cnt[2][wave] = wave_big; }
     __syncthreads();
-    rank = seen + before_in_wave;
+    // One pass per non-empty expert (the usual case): the jobs before this expert are the non-empty experts before it.
+    rank = seen + __popcll(m_act & ((1ull << lane) - 1ull));
     first_row = rows_seen + incl - sz;
     slab_act = 0; slab_rows = 0;
+    bool any_big = false;
     for (int w2 = 0; w2 < kThreads / 64; ++w2) {
       if (w2 < wave) { rank += wave_cnt[0][w2]; first_row += wave_cnt[1][w2]; }
       slab_act += wave_cnt[0][w2]; slab_rows += wave_cnt[1][w2];
+      any_big |= wave_cnt[2][w2] != 0;
+    }
+    if (any_big) {  // (the same in every thread) experts with several passes: count passes instead of experts
+      int incl_u = units;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) { const int up = __shfl_up(incl_u, d, 64); if (lane >= d) incl_u += up; }
+      __syncthreads();
+      if (lane == 63) wave_cnt[0][wave] = incl_u;
+      __syncthreads();
+      rank = seen + incl_u - units;
+      slab_act = 0;
+      for (int w2 = 0; w2 < kThreads / 64; ++w2) {
+        if (w2 < wave) rank += wave_cnt[0][w2];
+        slab_act += wave_cnt[0][w2];
+      }
     }
   };
   const bool one_slab = p.g <= kThreads;
   int sz0 = 0, rank0 = 0, first0 = 0;
-  int n_act = 0, total = 0;
+  int n_jobs = 0, total = 0;
   for (int base = 0; base < p.g; base += kThreads) {
     int sz, rank, first_row, sa, sr;
-    scan_slab(base, n_act, total, sz, rank, first_row, sa, sr);
+    scan_slab(base, n_jobs, total, sz, rank, first_row, sa, sr);
     if (base == 0) { sz0 = sz; rank0 = rank; first0 = first_row; }
-    n_act += sa; total += sr;
+    n_jobs += sa; total += sr;
   }
-  int C = n_act > 0 ? q.wgs / n_act : 1;
+  int C = n_jobs > 0 ? q.wgs / n_jobs : 1;
   C = imax(1, imin(imin(C, q.max_c), p.k / q.min_rows));
   if (blockIdx.x == 0 && tid == 0) { header->pieces = C; header->total_rows = imin(total, p.m); }
-  if (n_act == 0 || (int)blockIdx.x >= (q.wgs / C) * C) return;  // nothing to do / left-over work-groups
+  if (n_jobs == 0 || (int)blockIdx.x >= (q.wgs / C) * C) return;  // nothing to do / left-over work-groups
 
   const int c = blockIdx.x % C;
-  for (int want = blockIdx.x / C; want < n_act; want += q.wgs / C) {
+  for (int want = blockIdx.x / C; want < n_jobs; want += q.wgs / C) {
     // the `want`-th non-empty expert and the rows before it
     __syncthreads();  // job free again
     if (one_slab) {
-      if (sz0 > 0 && rank0 == want) { job[0] = tid; job[1] = first0; job[2] = sz0; }
+      if (sz0 > 0 && rank0 <= want && want < rank0 + (sz0 + RPP - 1) / RPP) {
+        const int done = (want - rank0) * RPP;  // rows of the expert that earlier passes take
+        job[0] = tid; job[1] = first0 + done; job[2] = imin(RPP, sz0 - done);
+      }
     } else {
       int seen = 0, rows_seen = 0;
       for (int base = 0; base < p.g; base += kThreads) {
         int sz, rank, first_row, sa, sr;
         scan_slab(base, seen, rows_seen, sz, rank, first_row, sa, sr);
-        if (sz > 0 && rank == want) { job[0] = base + tid; job[1] = first_row; job[2] = sz; }
+        if (sz > 0 && rank <= want && want < rank + (sz + RPP - 1) / RPP) {
+          const int done = (want - rank) * RPP;
+          job[0] = base + tid; job[1] = first_row + done; job[2] = imin(RPP, sz - done);
+        }
         seen += sa; rows_seen += sr;
       }
     }
@@ -610,8 +638,9 @@ __global__ __launch_bounds__(kThreads, 2) void gmm_rows_t_kernel(DecodeArgs p, i
   constexpr int EB = F8 ? 1 : 2;     // bytes per element of x and A
   constexpr int EPC = 16 / EB;       // elements per 16-byte chunk
   constexpr int XE = F8 ? 2 : 1;     // staged 16-byte entries per chunk and token row
-  __shared__ int32_t wave_cnt[2][kThreads / 64];
+  __shared__ int32_t wave_cnt[3][kThreads / 64];
   __shared__ int32_t job[3];
+  constexpr int RPP = RMAX;          // rows per pass
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   u32x4_t* xs = reinterpret_cast<u32x4_t*>(smem_raw);  // [RMAX rows][XE][chunk] x 16 bytes (8 bf16)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -619,31 +648,49 @@ __global__ __launch_bounds__(kThreads, 2) void gmm_rows_t_kernel(DecodeArgs p, i
   // which experts are non-empty and where their rows start (as in gmm_rows_kernel)
   auto scan_slab = [&](int base, int seen, int rows_seen, int& sz, int& rank, int& first_row, int& slab_act, int& slab_rows) {
     const int e = base + tid;
-    sz = e < p.g ? imax(p.group_sizes[e], 0) : 0;
+    sz = e < p.g ? imin(imax(p.group_sizes[e], 0), p.m) : 0;  // (no group has more than m rows that exist)
+    const int units = (sz + RPP - 1) / RPP;  // passes over this expert's weights, each a job of its own
     const unsigned long long m_act = __ballot(sz > 0);
-    const int before_in_wave = __popcll(m_act & ((1ull << lane) - 1ull));
+    const bool wave_big = __ballot(sz > RPP) != 0;  // some expert of this wave takes more than one pass
     int incl = sz;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) { const int up = __shfl_up(incl, d, 64); if (lane >= d) incl += up; }
     __syncthreads();
-    if (lane == 63) { wave_cnt[0][wave] = __popcll(m_act); wave_cnt[1][wave] = incl; }
+    if (lane == 63) { wave_cnt[0][wave] = __popcll(m_act); wave_cnt[1][wave] = incl; wave_cnt[2][wave] = wave_big; }
     __syncthreads();
-    rank = seen + before_in_wave;
+    // One pass per non-empty expert (the usual case): the jobs before this expert are the non-empty experts before it.
+    rank = seen + __popcll(m_act & ((1ull << lane) - 1ull));
     first_row = rows_seen + incl - sz;
     slab_act = 0; slab_rows = 0;
+    bool any_big = false;
     for (int w2 = 0; w2 < kThreads / 64; ++w2) {
       if (w2 < wave) { rank += wave_cnt[0][w2]; first_row += wave_cnt[1][w2]; }
       slab_act += wave_cnt[0][w2]; slab_rows += wave_cnt[1][w2];
+      any_big |= wave_cnt[2][w2] != 0;
+    }
+    if (any_big) {  // (the same in every thread) experts with several passes: count passes instead of experts
+      int incl_u = units;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) { const int up = __shfl_up(incl_u, d, 64); if (lane >= d) incl_u += up; }
+      __syncthreads();
+      if (lane == 63) wave_cnt[0][wave] = incl_u;
+      __syncthreads();
+      rank = seen + incl_u - units;
+      slab_act = 0;
+      for (int w2 = 0; w2 < kThreads / 64; ++w2) {
+        if (w2 < wave) rank += wave_cnt[0][w2];
+        slab_act += wave_cnt[0][w2];
+      }
     }
   };
   const bool one_slab = p.g <= kThreads;
   int sz0 = 0, rank0 = 0, first0 = 0;
-  int n_act = 0, total = 0;
+  int n_jobs = 0, total = 0;
   for (int base = 0; base < p.g; base += kThreads) {
     int sz, rank, first_row, sa, sr;
-    scan_slab(base, n_act, total, sz, rank, first_row, sa, sr);
+    scan_slab(base, n_jobs, total, sz, rank, first_row, sa, sr);
     if (base == 0) { sz0 = sz; rank0 = rank; first0 = first_row; }
-    n_act += sa; total += sr;
+    n_jobs += sa; total += sr;
   }
 
   // rows past sum(group_sizes) are zero: every work-group clears its share of them
@@ -653,12 +700,12 @@ __global__ __launch_bounds__(kThreads, 2) void gmm_rows_t_kernel(DecodeArgs p, i
     u32x4_t* tail = reinterpret_cast<u32x4_t*>(p.y + (size_t)t0 * p.n);
     for (size_t i = (size_t)blockIdx.x * kThreads + tid; i < words; i += (size_t)wgs * kThreads) tail[i] = u32x4_t{0, 0, 0, 0};
   }
-  if (n_act == 0) return;
-  int C = imax(1, imin(wgs / n_act, p.n / kTBlock));  // a piece holds at least one block of weight rows
+  if (n_jobs == 0) return;
+  int C = imax(1, imin(wgs / n_jobs, p.n / kTBlock));  // a piece holds at least one block of weight rows
   const int per = ((p.n + C - 1) / C + kTBlock - 1) / kTBlock * kTBlock;  // weight rows per piece (n % 8 == 0: whole blocks)
   C = (p.n + per - 1) / per;                          // pieces that hold any
-  const int experts_at_a_time = wgs / C;
-  if ((int)blockIdx.x >= experts_at_a_time * C) return;
+  const int jobs_at_a_time = wgs / C;
+  if ((int)blockIdx.x >= jobs_at_a_time * C) return;
   const int c = blockIdx.x % C;
   const int j_begin = c * per, j_end = imin(p.n, j_begin + per);
   const int chunks = p.k / EPC;                       // 16-byte chunks per weight row (k % EPC == 0)
@@ -666,16 +713,22 @@ __global__ __launch_bounds__(kThreads, 2) void gmm_rows_t_kernel(DecodeArgs p, i
   const int r_stride = npos * 64;                     // staged chunks per token row
   const unsigned char* xb = reinterpret_cast<const unsigned char*>(p.x);
 
-  for (int want = blockIdx.x / C; want < n_act; want += experts_at_a_time) {
+  for (int want = blockIdx.x / C; want < n_jobs; want += jobs_at_a_time) {
     __syncthreads();  // job free again
     if (one_slab) {
-      if (sz0 > 0 && rank0 == want) { job[0] = tid; job[1] = first0; job[2] = sz0; }
+      if (sz0 > 0 && rank0 <= want && want < rank0 + (sz0 + RPP - 1) / RPP) {
+        const int done = (want - rank0) * RPP;  // rows of the expert that earlier passes take
+        job[0] = tid; job[1] = first0 + done; job[2] = imin(RPP, sz0 - done);
+      }
     } else {
       int seen = 0, rows_seen = 0;
       for (int base = 0; base < p.g; base += kThreads) {
         int sz, rank, first_row, sa, sr;
         scan_slab(base, seen, rows_seen, sz, rank, first_row, sa, sr);
-        if (sz > 0 && rank == want) { job[0] = base + tid; job[1] = first_row; job[2] = sz; }
+        if (sz > 0 && rank <= want && want < rank + (sz + RPP - 1) / RPP) {
+          const int done = (want - rank) * RPP;
+          job[0] = base + tid; job[1] = first_row + done; job[2] = imin(RPP, sz - done);
+        }
         seen += sa; rows_seen += sr;
       }
     }
