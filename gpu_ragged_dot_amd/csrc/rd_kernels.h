@@ -35,6 +35,9 @@ struct GmmArgs {
   int max_parts;       // > 0: most pieces a tile is cut into, as the caller asked; 0: chosen from k
   int num_cus;         // tiles the device runs at a time (one work-group per compute unit)
   int main_grid;       // launch indices below this walk whole tiles (set by the launcher)
+  // order in which the blocks of the walk are dealt (see launch_sched_map; null: walk order)
+  const int32_t* block_order;
+  int n_blocks;
 };
 
 // dA[g, k, n] = x[rows of g, k]^T . dy[rows of g, n]
@@ -185,12 +188,27 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
     // With only a few rounds of tiles, blocks of the full size would leave some XCDs without work (180 tiles in blocks
     // of 32 occupy 6 of the 8): the blocks shrink so that every round deals one to each XCD.
     int per_block = p.group_m * p.group_n;
+    bool whole_blocks = true;
     if (live < 4 * p.num_cus) {
       const int rounds = (live + p.num_cus - 1) / p.num_cus;
-      per_block = imax(1, imin(per_block, (live + 8 * rounds - 1) / (8 * rounds)));
+      const int fewer = imax(1, imin(per_block, (live + 8 * rounds - 1) / (8 * rounds)));
+      whole_blocks = fewer == per_block;
+      per_block = fewer;
     }
     const int pos = blockIdx.x >> 3;
-    const int block = (pos / per_block) * 8 + (blockIdx.x & 7);
+    int block = (pos / per_block) * 8 + (blockIdx.x & 7);
+    // Groups much longer than a tile (matrix-core-bound tiles) and groups shorter than one (tiles that stream their
+    // group's weights) in one launch: their blocks are dealt evenly interleaved instead of in the order the groups come
+    // in, so that at any time some of an XCD's compute units multiply while the others stream (DeepSeek-V3 shape, dlhs:
+    // 1.63 -> 1.54 ms; all long groups first, or all short ones, is slower than either).  Same tiles, same results.
+    if (p.block_order && whole_blocks) {
+      const int n_long = uniform(p.block_order[0]), n_live = uniform(p.block_order[1]);
+      if (n_long > 0 && n_long < n_live && block < n_live) {
+        const int before = (int)((long long)block * n_long / n_live);           // long blocks dealt before this one
+        const int upto = (int)((long long)(block + 1) * n_long / n_live);
+        block = uniform(upto > before ? p.block_order[2 + before] : p.block_order[2 + p.n_blocks - 1 - (block - before)]);
+      }
+    }
     t = block * per_block + pos % per_block;
     if (t >= p.U * p.n_tiles) return;
     if (t >= sp.first_tile && t < live) return;  // computed in pieces by the appended work-groups

@@ -47,7 +47,9 @@ __global__ __launch_bounds__(kSchedThreads) void sched_map_kernel(const int32_t*
                                                                   int32_t* __restrict__ tile2it,
                                                                   int32_t* __restrict__ total_tiles,
                                                                   int32_t* __restrict__ counters, int n_counters,
-                                                                  int32_t* __restrict__ tile2band, int band_rows) {
+                                                                  int32_t* __restrict__ tile2band, int band_rows,
+                                                                  int32_t* __restrict__ block_order, int n_blocks,
+                                                                  int per_block, int n_tiles, int long_rows) {
   // arrival counters of the K-split tiles of the launch that follows start at zero
   for (int i = threadIdx.x; i < n_counters; i += kSchedThreads) counters[i] = 0;
   __shared__ uint32_t wave_a[kSchedWaves], wave_b[kSchedWaves];
@@ -100,6 +102,33 @@ __global__ __launch_bounds__(kSchedThreads) void sched_map_kernel(const int32_t*
     if (tile2band) tile2band[t] = (t << kBandShift) | 1;  // the slots that zero the rows past sum(group_sizes): one-tile bands
   }
   if (tid == 0) *total_tiles = (int32_t)carry_tiles;  // :89
+
+  if (block_order) {
+    // The blocks of the gmm tile walk, sorted into those of long groups (from the front) and the others (from the back);
+    // a block is judged by the group of its first position.
+    __threadfence_block();
+    __syncthreads();  // the map above is complete
+    const int total = imax(imin((int32_t)carry_tiles, U), 0);
+    const int live_blocks = imin((int)(((long long)total * n_tiles + per_block - 1) / per_block), n_blocks);
+    int32_t* order = block_order + 2;
+    uint32_t carry_l = 0, carry_s = 0;
+    for (int base = 0; base < live_blocks; base += kSchedThreads) {
+      const int b = base + tid;
+      bool is_long = false, is_short = false;
+      if (b < live_blocks) {
+        const int slot = imin((int)(((long long)b * per_block) / n_tiles), total - 1);
+        is_long = gs[tile2group[slot]] > long_rows;
+        is_short = !is_long;
+      }
+      uint32_t a = is_long, c = is_short, ta, tc;
+      block_scan2(a, c, ta, tc, wave_a, wave_b);
+      if (is_long) order[carry_l + a - 1] = b;
+      if (is_short) order[n_blocks - 1 - (int)(carry_s + c - 1)] = b;
+      carry_l += ta;
+      carry_s += tc;
+    }
+    if (tid == 0) { block_order[0] = (int32_t)carry_l; block_order[1] = (int32_t)(carry_l + carry_s); }
+  }
 }
 
 template <typename T>
@@ -139,12 +168,15 @@ int launch_stream_read(hipStream_t s, const void* src, size_t bytes, size_t bloc
 
 int launch_sched_map(hipStream_t s, const int32_t* gs, int g, int m, int chunk, int32_t* group_offsets,
                      int32_t* tile2group, int32_t* tile2it, int32_t* total_tiles, int32_t* counters, int n_counters,
-                     int32_t* tile2band, int band_rows) {
+                     int32_t* tile2band, int band_rows, int32_t* block_order, int n_blocks, int per_block, int n_tiles,
+                     int long_rows) {
   const int U = (m + chunk - 1) / chunk + g;  // gpu_ragged_dot.py:77
   if (band_rows < 1) band_rows = 1;
   if (band_rows > kBandMaxRows) band_rows = kBandMaxRows;
   hipLaunchKernelGGL(sched_map_kernel, dim3(1), dim3(kSchedThreads), 0, s, gs, g, U, chunk, group_offsets,
-                     tile2group, tile2it, total_tiles, counters, counters ? n_counters : 0, tile2band, band_rows);
+                     tile2group, tile2it, total_tiles, counters, counters ? n_counters : 0, tile2band, band_rows,
+                     n_blocks > 0 ? block_order : nullptr, n_blocks, per_block > 0 ? per_block : 1, n_tiles > 0 ? n_tiles : 1,
+                     long_rows);
   return (int)hipGetLastError();
 }
 

@@ -182,6 +182,48 @@ def test_tgmm_group_length_classes(vid, vname, group_m):
     assert np.array_equal(out, want)
 
 
+@pytest.mark.parametrize("trans_rhs", [False, True], ids=["A", "At"])
+@pytest.mark.parametrize("vname,walk", [("w256x256x32_w2x2_s5", (4, 8)), ("w256x256x32_w2x2_s5", (2, 4)),
+                                        ("p256x256x32_w2x4_s4", (3, 5)), ("d128x128x32_w2x2_s3", (4, 8))])
+def test_interleaved_block_order_is_transparent(vname, walk, trans_rhs):
+    """With several rounds of tiles and room in the workspace, the blocks of the tile walk that belong to groups longer
+    than the streaming routines serve are dealt interleaved with the others'.  The same tiles are computed: the result
+    must equal, bit for bit, that of a call whose workspace holds the scheduling map and nothing else (blocks in walk
+    order), and the oracle's within the usual bounds.  Long and short groups in every order, empty ones, a zero tail."""
+    print(f"interleaved block order {vname} walk={walk} trans_rhs={trans_rhs}", flush=True)
+    k, n = 72, 4096
+    rng = np.random.default_rng(5)
+    lens = list(rng.integers(1, 120, size=58)) + [0, 0, 0, 700, 1300, 257, 129, 128, 530]
+    rng.shuffle(lens)
+    gs = np.array(lens, np.int32)
+    g = len(lens)
+    m = int(gs.sum()) + 300
+    lhs = oracle.round_to(rng.standard_normal((m, k)).astype(np.float32), "bfloat16")
+    rhs = oracle.round_to((rng.standard_normal((g, k, n)) / k ** 0.5).astype(np.float32), "bfloat16")
+    vid = [v.id for v in _capi.variants() if v.name.decode() == vname][0]
+    bm = [v.tile_m for v in _capi.variants() if v.id == vid][0]
+    plan = _capi.Plan(vid, walk[0], 0, walk[1], split_k=-1)
+    x, A, gsd = util.bf16_dev(lhs), util.bf16_dev(rhs), torch.from_numpy(gs).cuda()
+    Ad = A.mT.contiguous() if trans_rhs else A
+    U = -(-m // bm) + g
+    assert U * (n // 256) >= 1024 and (-(-gs // bm)).sum() * (n // 256) >= 1024   # several rounds of live tiles
+    map_only = -(-((g + 3 * U + 1) * 4) // 256) * 256
+    outs = []
+    for ws_bytes in (_capi.lib.rd_gmm_workspace_bytes(m, g, ctypes.byref(plan)), map_only):
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+        y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        rc = _capi.lib.rd_gmm(torch.cuda.current_stream().cuda_stream, x.data_ptr(), Ad.data_ptr(), gsd.data_ptr(),
+                              y.data_ptr(), m, k, n, g, int(trans_rhs), _capi.RD_DTYPE_BF16, ctypes.byref(plan),
+                              ws.data_ptr(), ws_bytes)
+        assert rc == _capi.RD_OK, _capi.lib.rd_last_error()
+        torch.cuda.synchronize()
+        outs.append(y)
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+    got = util.to_np(outs[0])
+    util.assert_close_rows(got, oracle.gmm(lhs, rhs, gs), int(gs.sum()), util.BF16_EPS, "interleaved")
+    assert not np.any(got[int(gs.sum()):])
+
+
 def _split_variants():
     return [(v.id, v.name.decode()) for v in _capi.variants() if v.dtype == _capi.RD_DTYPE_BF16 and v.direct_to_lds]
 
