@@ -156,9 +156,16 @@ def test_default_plan_scales_the_tile_with_the_problem():
         assert tile(op, 32768, 7168, 2048, 256) == (256, 256)
     assert tile(_capi.OP_GMM, 6144, 6144, 1536, 6) == (256, 256)      # few tiles, long contraction
     assert tile(_capi.OP_GMM, 65536, 512, 512, 64) == (128, 256)      # short contraction: two work-groups per compute unit hide the tile set-up
-    assert tile(_capi.OP_GMM_TRANS, 8192, 4096, 256, 16) == (128, 128)
+    assert tile(_capi.OP_GMM_TRANS, 8192, 4096, 256, 16) == (64, 64)      # 144 tiles of 128 x 128: too few
     assert tile(_capi.OP_TGMM, 4096, 1024, 1024, 8) == (128, 128)
     assert max(tile(_capi.OP_GMM, 2048, 4096, 512, 4)) <= 128 and max(tile(_capi.OP_GMM, 256, 64, 64, 4)) <= 128
+    # few 128 x 128 tiles and a moderate contraction: four times as many 64 x 64 tiles, walked in blocks of 16
+    assert tile(_capi.OP_GMM, 256, 4096, 4096, 2) == (64, 64) and tile(_capi.OP_GMM, 1280, 1280, 1280, 10) == (64, 64)
+    p = _capi.default_plan(_capi.OP_GMM_TRANS, 1024, 2048, 512, 4)
+    assert (vs[p.variant].tile_m, vs[p.variant].tile_n, p.group_m, p.group_n) == (64, 64, 4, 4)
+    assert tile(_capi.OP_GMM_TRANS, 1536, 8192, 1024, 3) == (128, 128)   # ... but not with a contraction of 8192
+    # trans_rhs, long contraction, under a round of 256 x 256 tiles: the eight-wave 256 x 256 core and its K-split
+    assert vs[_capi.default_plan(_capi.OP_GMM_TRANS, 512, 8192, 8192, 1).variant].name.decode() == "p256x256x32_w2x4_s4"
     assert tile(_capi.OP_GMM, 8192, 4096, 4096, 8, dtype=_capi.RD_DTYPE_F32) == (128, 128)
     assert tile(_capi.OP_GMM, 512, 256, 256, 4, dtype=_capi.RD_DTYPE_F32) == (64, 64)
 
