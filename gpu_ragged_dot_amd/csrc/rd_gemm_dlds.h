@@ -80,7 +80,9 @@ struct DldsLoader {
   int voff[PER];          // per-lane byte offset of each load
   int kcol;               // K-major: contraction offset (elements) of this lane's chunk, for the tail predicate
 
-  __device__ __forceinline__ void init(const bf16_bits* p, int ld, int lim, int klen, int wave, int lane) {
+  // (init and advance are plain integer arithmetic and also run on the host: tests/host_checks/loader_bounds.hip walks
+  // every load of every slab through them and checks it against the operand's window)
+  __host__ __device__ __forceinline__ void init(const bf16_bits* p, int ld, int lim, int klen, int wave, int lane) {
     base = p;
     if (KMAJOR) {
       records = ((lim - 1) * ld + klen) * 2;
@@ -120,7 +122,7 @@ struct DldsLoader {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(lds + (wave + NW * j) * 1024), 16, off, 0, 0, AUX);
   }
 
-  __device__ __forceinline__ void advance() {
+  __host__ __device__ __forceinline__ void advance() {
     base = reinterpret_cast<const bf16_bits*>(reinterpret_cast<const unsigned char*>(base) + step_bytes);
     records -= step_bytes;  // stays positive for every slab that is issued
   }
