@@ -198,16 +198,15 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
     const int pos = blockIdx.x >> 3;
     int block = (pos / per_block) * 8 + (blockIdx.x & 7);
     // Groups much longer than a tile (matrix-core-bound tiles) and groups shorter than one (tiles that stream their
-    // group's weights) in one launch: their blocks are dealt evenly interleaved instead of in the order the groups come
-    // in, so that at any time some of an XCD's compute units multiply while the others stream (DeepSeek-V3 shape, dlhs:
-    // 1.63 -> 1.54 ms; all long groups first, or all short ones, is slower than either).  Same tiles, same results.
+    // group's weights) in one launch: their blocks are dealt interleaved instead of in the order the groups come in, so
+    // that at any time some of every XCD's compute units multiply while the others stream (DeepSeek-V3 shape, dlhs:
+    // 1.63 -> 1.55 ms; all long groups first, or all short ones, is slower than either).  Same tiles, same results.
     if (p.block_order && whole_blocks) {
       const int n_long = uniform(p.block_order[0]), n_live = uniform(p.block_order[1]);
-      if (n_long > 0 && n_long < n_live && block < n_live) {
-        const int before = (int)((long long)block * n_long / n_live);           // long blocks dealt before this one
-        const int upto = (int)((long long)(block + 1) * n_long / n_live);
-        block = uniform(upto > before ? p.block_order[2 + before] : p.block_order[2 + p.n_blocks - 1 - (block - before)]);
-      }
+      bool from_long;
+      int rank;
+      if (interleaved_slot(block, n_long, n_live, &from_long, &rank))
+        block = uniform(p.block_order[from_long ? 2 + rank : 2 + p.n_blocks - 1 - rank]);
     }
     t = block * per_block + pos % per_block;
     if (t >= p.U * p.n_tiles) return;
