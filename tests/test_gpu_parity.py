@@ -600,7 +600,8 @@ def test_float32_every_tile_shape(shape):
 
 def test_streaming_default_with_all_rows_in_one_group():
     """The shape-only default picks the streaming kernel for m <= 4 g; the shape cannot see that all rows sit in one
-    group, whose weights are then streamed once per 8 rows.  Slow (the header says so) but it must be right."""
+    group, whose weights are then streamed once per 8 rows - every such pass a job of its own, spread over the
+    work-groups."""
     print("streaming default, all rows in one group", flush=True)
     m, k, n, g = 256, 2048, 768, 128
     assert _capi.default_plan(_capi.OP_GMM, m, k, n, g).decode_nb == _capi.RD_DECODE_ROWS
