@@ -115,9 +115,10 @@ int rd_sched_map_len(int m, int g, int chunk_m);
  *   A is [g, k, n] (trans_rhs = 0) or [g, n, k] (trans_rhs = 1, gpu_ragged_dot.py:139-144, :190).
  *   Rows of group i are [offset_i, offset_i + group_sizes[i]); rows >= sum(group_sizes) of y are set to zero
  *   (:155-165) -- also when every group is empty.  Groups that would run past m are clipped to m.
- * Workspace: rd_gmm_workspace_bytes() bytes, 256-byte aligned; holds the scheduling map and, unless the plan says
- * split_k = -1, fp32 partial sums (64 MiB for the 256 x 256 tiles).  A workspace that only has room for the map
- * (the size returned for a plan with split_k = -1) is accepted: the call then runs without the K-split. */
+ * Workspace: rd_gmm_workspace_bytes() bytes, 256-byte aligned; holds the scheduling map, 64 KiB for the order in which
+ * the tile walk's blocks are dealt (long groups' among short groups') and, unless the plan says split_k = -1, fp32
+ * partial sums (64 MiB for the 256 x 256 tiles).  A smaller workspace that has room for the map is accepted: the call
+ * then runs without the K-split and, if the order does not fit either, in plain walk order - same results. */
 size_t rd_gmm_workspace_bytes(int m, int g, const rd_plan* plan /* host, may be NULL */);
 int rd_gmm(void* stream, const void* x, const void* A, const int32_t* group_sizes, void* y, int m, int k, int n,
            int g, int trans_rhs, int dtype, const rd_plan* plan /* host, may be NULL */, void* workspace,
@@ -145,7 +146,8 @@ int rd_tgmm_sharded(void* stream, const void* x, const void* dy, const int32_t* 
  * caller's workspace (the scheduling map, the streaming kernel's partial sums) lives in a buffer of
  * rd_gmm_noalloc_scratch_bytes() = 4 MiB built into the library, one copy per device, held until the process ends.
  * The call allocates and frees nothing.  Limits: the scheduling map must fit (rd_gmm_workspace_bytes(m, g, plan with
- * split_k = -1) <= 4 MiB, i.e. roughly m / 16 + g <= 349 000), otherwise RD_ERR_WORKSPACE; the K-split is never used.
+ * split_k = -1) <= 4 MiB, i.e. roughly 12 (m / 16) + 16 g bytes <= 4 MiB - 64 KiB: 5.5 M rows with a few hundred groups),
+ * otherwise RD_ERR_WORKSPACE; the K-split is never used.
  * All calls on one device share that device's buffer: calls that overlap on one device (different streams, or
  * different threads without stream ordering between them) race; calls ordered on one stream do not. */
 size_t rd_gmm_noalloc_scratch_bytes(void);
