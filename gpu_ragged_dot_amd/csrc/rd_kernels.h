@@ -51,6 +51,7 @@ struct TgmmArgs {
   int g_first;     // dA[i] belongs to group g_first + i of group_sizes / group_offsets
   int k_tiles, n_tiles;  // ceil(k / BM), ceil(n / BN)
   int group_m;
+  const int32_t* group_order;  // null, or the records of the order in which the launch visits the groups (launch_sched_map)
 };
 
 // A value every lane holds identically, moved to a scalar register.
@@ -310,9 +311,20 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void tgmm_kernel(TgmmArgs p
   const int per_group = p.k_tiles * p.n_tiles;
   const int quota = (per_group + 7) >> 3;  // tiles of one group per XCD
   const int xcd = blockIdx.x & 7, pos = blockIdx.x >> 3;
-  const int gi = pos / quota;
-  const int t = ((xcd + gi) & 7) * quota + (pos - gi * quota);
-  if (gi >= p.g || t >= per_group) return;
+  const int slot = pos / quota;
+  if (slot >= p.g) return;
+  // groups are visited by falling size class, so that tiles of about equal duration run side by side; the record of
+  // a position holds the group, its first row and its row count
+  int gi = slot, row0, rows;
+  if (p.group_order) {
+    const int32_t* rec = p.group_order + 4 * (size_t)slot;
+    gi = uniform(rec[0]); row0 = uniform(rec[1]); rows = uniform(rec[2]);
+  } else {
+    row0 = uniform(p.group_offsets[slot + p.g_first]);
+    rows = uniform(p.group_sizes[slot + p.g_first]);
+  }
+  const int t = ((xcd + slot) & 7) * quota + (pos - slot * quota);
+  if (gi < 0 || gi >= p.g || t >= per_group) return;
   int ri, cj;
   band_walk(t, p.k_tiles, p.n_tiles, p.group_m, ri, cj);
 
@@ -321,8 +333,6 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void tgmm_kernel(TgmmArgs p
   typedef typename OutOf<C>::type O;
   O* Op = static_cast<O*>(p.dA) + (size_t)gi * p.k * p.n + (size_t)kk0 * p.n + col0;
 
-  const int row0 = uniform(p.group_offsets[gi + p.g_first]);
-  int rows = uniform(p.group_sizes[gi + p.g_first]);
   rows = imin(rows, p.m - row0);
   if (rows <= 0 || row0 < 0) {  // empty group: its slice of dA is zero
     zero_tile<C::NT, C::VEC, O>(Op, p.n, krows, cols);

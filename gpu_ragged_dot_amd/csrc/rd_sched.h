@@ -19,10 +19,19 @@ constexpr int kBandMaxRows = (1 << kBandShift) - 1;
 // tiles are bound by the matrix cores - and shorter ones - whose tiles stream their group's weights - share a launch:
 //   [0] blocks of long groups L, [1] live blocks L + S, [2 ..] the long groups' blocks in walk order from the front,
 //   the others' from the back (last entry first).  interleaved_slot() says which list a position of the launch takes from.
+// `group_order` (may be null; order_count records of 4 words): for tgmm, the groups [order_first, order_first +
+// order_count) of group_sizes, numbered from 0, listed by falling size class (bit length of the row count: 0, 1, 2-3,
+// 4-7, ...) and by index within a class; a record holds the group's number, first row and row count (one load per tile:
+// looking the group up first and its rows after costs a short group's tile a second round trip, 2 % of the launch).  A tgmm launch that visits the groups in this order runs tiles of about equal duration side
+// by side (DeepSeek-V3 shape, 256 groups of 0 to 7099 rows: 1.97 -> 1.92 ms; with the groups also stored in that order
+// 1.90; an exact sort by rows gives the same, classes of 64 or 128 rows half of it or nothing, long groups merely moved
+// to the front nothing).  Where two groups' tiles share an XCD the order the groups come in mixes long and short
+// tiles and is the better one (128 groups with Zipf lengths, k 2048, n 4096: 0.84 -> 0.88 ms), hence an option of the plan.
 int launch_sched_map(hipStream_t s, const int32_t* group_sizes, int g, int m, int chunk, int32_t* group_offsets,
                      int32_t* tile2group, int32_t* tile2it, int32_t* total_tiles, int32_t* counters = nullptr,
                      int n_counters = 0, int32_t* tile2band = nullptr, int band_rows = 1, int32_t* block_order = nullptr,
-                     int n_blocks = 0, int per_block = 1, int n_tiles = 1, int long_rows = 0);
+                     int n_blocks = 0, int per_block = 1, int n_tiles = 1, int long_rows = 0,
+                     int32_t* group_order = nullptr, int order_first = 0, int order_count = 0);
 
 // Which block the i-th block position of a gmm launch takes from the two lists of block_order.  Positions are dealt to
 // the 8 XCDs round-robin (position i runs on XCD i mod 8), so the launch is a sequence of rounds of 8.  The long groups'

@@ -41,6 +41,9 @@ __device__ __forceinline__ void block_scan2(uint32_t& a, uint32_t& b, uint32_t& 
   __syncthreads();
 }
 
+constexpr int kSizeClasses = 33;
+__device__ __forceinline__ int size_class(int32_t rows) { return rows <= 0 ? 0 : 32 - __clz(rows); }
+
 __global__ __launch_bounds__(kSchedThreads) void sched_map_kernel(const int32_t* __restrict__ gs, int g, int U,
                                                                   int chunk, int32_t* __restrict__ group_offsets,
                                                                   int32_t* __restrict__ tile2group,
@@ -49,7 +52,9 @@ __global__ __launch_bounds__(kSchedThreads) void sched_map_kernel(const int32_t*
                                                                   int32_t* __restrict__ counters, int n_counters,
                                                                   int32_t* __restrict__ tile2band, int band_rows,
                                                                   int32_t* __restrict__ block_order, int n_blocks,
-                                                                  int per_block, int n_tiles, int long_rows) {
+                                                                  int per_block, int n_tiles, int long_rows,
+                                                                  int32_t* __restrict__ group_order, int order_first,
+                                                                  int order_count) {
   // arrival counters of the K-split tiles of the launch that follows start at zero
   for (int i = threadIdx.x; i < n_counters; i += kSchedThreads) counters[i] = 0;
   __shared__ uint32_t wave_a[kSchedWaves], wave_b[kSchedWaves];
@@ -129,6 +134,49 @@ __global__ __launch_bounds__(kSchedThreads) void sched_map_kernel(const int32_t*
     }
     if (tid == 0) { block_order[0] = (int32_t)carry_l; block_order[1] = (int32_t)(carry_l + carry_s); }
   }
+  if (group_order) {
+    __threadfence_block();  // group_offsets, written above by other threads of this work-group, are read below
+    // tgmm: groups [order_first, order_first + order_count) listed by falling size class (bit length of the row count:
+    // 0, 1, 2-3, 4-7, ...), groups of one class in index order - a stable counting sort over 33 classes.
+    __shared__ int32_t cls_base[kSizeClasses], cls_wave[kSchedWaves][kSizeClasses];
+    __syncthreads();
+    if (tid < kSizeClasses) cls_base[tid] = 0;
+    __syncthreads();
+    for (int i = tid; i < order_count; i += kSchedThreads) atomicAdd(&cls_base[size_class(gs[order_first + i])], 1);
+    __syncthreads();
+    if (tid == 0) {
+      int32_t run = 0;
+      for (int c = kSizeClasses - 1; c >= 0; --c) { const int32_t cnt = cls_base[c]; cls_base[c] = run; run += cnt; }
+    }
+    __syncthreads();
+    const int lane = tid & 63, wave = tid >> 6;
+    for (int base = 0; base < order_count; base += kSchedThreads) {
+      const int i = base + tid;
+      const int c = i < order_count ? size_class(gs[order_first + i]) : -1;
+      int rank = 0;
+      for (int cc = 0; cc < kSizeClasses; ++cc) {
+        const unsigned long long mask = __ballot(c == cc);
+        if (c == cc) rank = __popcll(mask & ((1ull << lane) - 1ull));
+        if (lane == 0) cls_wave[wave][cc] = __popcll(mask);
+      }
+      __syncthreads();
+      if (c >= 0) {
+        int32_t before = cls_base[c];
+        for (int w = 0; w < wave; ++w) before += cls_wave[w][c];
+        // one record per position: the group, its first row and its row count, so that a tile of the launch finds all
+        // three with a single load
+        int32_t* rec = group_order + 4 * (before + rank);
+        rec[0] = i; rec[1] = group_offsets[order_first + i]; rec[2] = gs[order_first + i]; rec[3] = 0;
+      }
+      __syncthreads();
+      if (tid < kSizeClasses) {
+        int32_t tot = 0;
+        for (int w = 0; w < kSchedWaves; ++w) tot += cls_wave[w][tid];
+        cls_base[tid] += tot;
+      }
+      __syncthreads();
+    }
+  }
 }
 
 template <typename T>
@@ -169,14 +217,14 @@ int launch_stream_read(hipStream_t s, const void* src, size_t bytes, size_t bloc
 int launch_sched_map(hipStream_t s, const int32_t* gs, int g, int m, int chunk, int32_t* group_offsets,
                      int32_t* tile2group, int32_t* tile2it, int32_t* total_tiles, int32_t* counters, int n_counters,
                      int32_t* tile2band, int band_rows, int32_t* block_order, int n_blocks, int per_block, int n_tiles,
-                     int long_rows) {
+                     int long_rows, int32_t* group_order, int order_first, int order_count) {
   const int U = (m + chunk - 1) / chunk + g;  // gpu_ragged_dot.py:77
   if (band_rows < 1) band_rows = 1;
   if (band_rows > kBandMaxRows) band_rows = kBandMaxRows;
   hipLaunchKernelGGL(sched_map_kernel, dim3(1), dim3(kSchedThreads), 0, s, gs, g, U, chunk, group_offsets,
                      tile2group, tile2it, total_tiles, counters, counters ? n_counters : 0, tile2band, band_rows,
                      n_blocks > 0 ? block_order : nullptr, n_blocks, per_block > 0 ? per_block : 1, n_tiles > 0 ? n_tiles : 1,
-                     long_rows);
+                     long_rows, order_count > 0 ? group_order : nullptr, order_first, order_count);
   return (int)hipGetLastError();
 }
 

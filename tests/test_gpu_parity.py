@@ -182,6 +182,48 @@ def test_tgmm_group_length_classes(vid, vname, group_m):
     assert np.array_equal(out, want)
 
 
+@pytest.mark.parametrize("vname", [None, "p256x256x32_w2x4_s4", "d128x128x32_w2x2_s3", "t64x64x64_w2x2"])
+@pytest.mark.parametrize("g_first,g_local", [(0, 30), (7, 16)])
+def test_tgmm_group_order_is_transparent(vname, g_first, g_local):
+    """With plan.group_n = 1 and room for it in the workspace a tgmm launch visits the groups by falling size class.
+    The same tiles are computed: the result must equal, bit for bit, that of a call whose workspace holds the row
+    offsets only, and the oracle's; also for a slice of the groups (group_offset)."""
+    print(f"tgmm group order {vname} groups [{g_first}, {g_first}+{g_local})", flush=True)
+    k, n = 264, 520
+    lens = [0, 1, 31, 32, 33, 64, 65, 96, 97, 127, 128, 129, 160, 300, 0, 0, 7, 1100, 5, 0, 40, 200, 95, 2, 0, 64, 31, 513, 96, 33]
+    rng = np.random.default_rng(23)
+    gs = np.array(lens, np.int32)
+    g = len(lens)
+    m = int(gs.sum()) + 21
+    lhs = oracle.round_to(rng.standard_normal((m, k)).astype(np.float32), "bfloat16")
+    dout = oracle.round_to(rng.standard_normal((m, n)).astype(np.float32), "bfloat16")
+    plan = _capi.Plan(-1 if vname is None else [v.id for v in _capi.variants() if v.name.decode() == vname][0], 3, 0, 1)
+    pref = ctypes.byref(plan)
+    x, d, gsd = util.bf16_dev(lhs), util.bf16_dev(dout), torch.from_numpy(gs).cuda()
+    full = _capi.lib.rd_tgmm_workspace_bytes(m, g, pref)
+    offsets_only = -(-((g + 3 * (g + 1) + 1) * 4) // 256) * 256
+    assert full >= offsets_only + 16 * g
+    stream = torch.cuda.current_stream().cuda_stream
+    outs = []
+    for ws_bytes in (full, offsets_only):
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+        dA = torch.full((g_local, k, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        if (g_first, g_local) == (0, g):
+            rc = _capi.lib.rd_tgmm(stream, x.data_ptr(), d.data_ptr(), gsd.data_ptr(), dA.data_ptr(), m, k, n, g,
+                                   _capi.RD_DTYPE_BF16, pref, ws.data_ptr(), ws_bytes)
+        else:
+            rc = _capi.lib.rd_tgmm_sharded(stream, x.data_ptr(), d.data_ptr(), gsd.data_ptr(), dA.data_ptr(), m, k, n, g,
+                                           g_first, g_local, _capi.RD_DTYPE_BF16, pref, ws.data_ptr(), ws_bytes)
+        assert rc == _capi.RD_OK, _capi.lib.rd_last_error()
+        torch.cuda.synchronize()
+        outs.append(dA)
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+    got = util.to_np(outs[0])
+    sl = slice(g_first, g_first + g_local)
+    util.assert_close_groups(got, oracle.tgmm(lhs, dout, gs)[sl], gs[sl] != 0, util.TGMM_BF16_EPS, "tgmm group order")
+    assert not np.any(got[gs[sl] == 0])
+
+
 @pytest.mark.parametrize("trans_rhs", [False, True], ids=["A", "At"])
 @pytest.mark.parametrize("vname,walk", [("w256x256x32_w2x2_s5", (4, 8)), ("w256x256x32_w2x2_s5", (2, 4)),
                                         ("p256x256x32_w2x4_s4", (3, 5)), ("d128x128x32_w2x2_s3", (4, 8))])
