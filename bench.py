@@ -330,6 +330,79 @@ def dense_gemm_context(torch):
                     "dout.W^T (dlhs layout), x^T.dout (drhs layout)", **out}, own
 
 
+def tile_boundary_context(torch):
+    """What everything between two tiles of a compute unit costs (epilogue, the next work-group's look-ups and prologue,
+    the ring filling up again): the FLOPs of one dense Mixtral product as ONE group of 16384 rows on N(0,1) data, with
+    the contraction lengthened and the output narrowed so that a compute unit runs 4 (14 for the forward layout), 2 (4)
+    or a single 256 x 256 tile.  With one tile per compute unit there are no boundaries left: the difference to the
+    first column bounds what a persistent tile-to-tile schedule could gain on this data."""
+    from gpu_ragged_dot_amd import _capi, ops, planner
+
+    m = 16384
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    vid = planner.variant_id("w256x256x32_w2x2_s5")
+    plan = _capi.Plan(vid, 4, 0, 8, -1)
+    one = torch.tensor([m], dtype=torch.int32, device="cuda")
+    out = {"what": "w256x256x32_w2x2_s5, one group of 16384 rows, 1.924e12 FLOP per launch, N(0,1) data, K-split off; "
+                   "key = tiles per compute unit"}
+    shapes = {"dlhs_layout": (True, ((14336, 4096), (28672, 2048), (57344, 1024))),
+              "forward_layout": (False, ((4096, 14336), (14336, 4096), (57344, 1024)))}
+    for label, (trans, kns) in shapes.items():
+        res = {}
+        for k, n in kns:
+            x = torch.randn((m, k), generator=gen, device="cuda").to(torch.bfloat16)
+            a = (torch.randn((1, n, k) if trans else (1, k, n), generator=gen, device="cuda") / k ** 0.5).to(torch.bfloat16)
+            fn = lambda: ops._gmm_fwd(x, a, one, **HP, acc_dtype=torch.float32, trans_rhs=trans, plan=plan)
+            for _ in range(3):
+                fn()
+            ms = _event_ms(fn, 10, torch)
+            res[str((m // 256) * (n // 256) // 256)] = {"k": k, "n": n, "ms": ms, "TFLOP/s": 2.0 * m * k * n / (ms * 1e-3) / 1e12}
+            del x, a
+        out[label] = res
+    return out
+
+
+def schedule_context(torch):
+    """The two orderings the scheduling-map kernel builds, each against the plain order on the DeepSeek-V3 workload in
+    this process: gmm trans_rhs (dlhs) with the blocks of long and short groups dealt interleaved (what a call with the
+    full workspace does) against the walk order (the same call through the C ABI with a workspace that holds only the
+    scheduling map); tgmm (drhs) with the groups visited by falling size class (plan group_n = 1, the tuned plan) against
+    the order they come in (group_n = 0)."""
+    import ctypes
+
+    from gpu_ragged_dot_amd import _capi, ops, planner, workloads
+
+    name = "deepseek_fwd_bwd"
+    x, A, dout, gs = workloads.make_inputs(name)
+    w = workloads.WORKLOADS[name]
+    m, k, n, g = w.m, w.k, w.n, w.g
+    out = {"what": "deepseek_fwd_bwd, ms per launch"}
+    # dlhs through the C ABI: y[m, k] = dout[m, n] . A[g, k, n]^T, i.e. rd_gmm(trans_rhs) with contraction n
+    plan = planner.select_plan(_capi.OP_GMM_TRANS, m, n, k, g)
+    y = torch.empty((m, k), dtype=torch.bfloat16, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    tile_m = [v.tile_m for v in _capi.variants() if v.id == plan.variant][0]
+    units = -(-m // tile_m) + g
+    map_only = -(-((g + 3 * units + 1) * 4) // 256) * 256
+    full = _capi.lib.rd_gmm_workspace_bytes(m, g, ctypes.byref(plan))
+    for label, nbytes in (("dlhs_blocks_interleaved", full), ("dlhs_blocks_in_walk_order", map_only)):
+        ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        fn = lambda: _capi.check(_capi.lib.rd_gmm(stream, dout.data_ptr(), A.data_ptr(), gs.data_ptr(), y.data_ptr(), m, n, k, g,
+                                                   1, _capi.RD_DTYPE_BF16, ctypes.byref(plan), ws.data_ptr(), nbytes))
+        for _ in range(3):
+            fn()
+        out[label] = _event_ms(fn, 20, torch)
+    tuned = planner.select_plan(_capi.OP_TGMM, m, k, n, g)
+    for label, gn in (("drhs_groups_by_size_class", 1), ("drhs_groups_as_they_come", 0)):
+        p2 = _capi.Plan(tuned.variant, tuned.group_m, 0, gn, 0)
+        fn = lambda: ops._tgmm_fwd(x, dout, gs, **HP, acc_dtype=torch.float32, plan=p2)
+        for _ in range(3):
+            fn()
+        out[label] = _event_ms(fn, 20, torch)
+    out["plans"] = {"dlhs": _plan_text(plan, planner), "drhs": _plan_text(tuned, planner)}
+    return out
+
+
 def float8_context(torch):
     """The Mixtral-shaped products with float8 e4m3fn operands (bf16 out, fp32 accumulation): forward products only - the
     library has no float8 VJP - so this is context beside the bf16 metric, not a configuration of it."""
@@ -490,6 +563,7 @@ def main():
         out["context"] = {"dense_gemm": vendor_dense, "own_dense_gemm": own_dense, "sustained_headline_step": out.pop("sustained", None),
                           "decode_bare_stream": configs["decode"].pop("bare_stream", None),
                           "decode_trans_rhs": configs["decode"].pop("trans_rhs", None),
+                          "tiles_per_compute_unit": tile_boundary_context(torch), "schedule_orders": schedule_context(torch),
                           "float8_mixtral_products": float8_context(torch), "cpu": cpu_model(),
                           "device": torch.cuda.get_device_name(0)}
     print(json.dumps(out))
