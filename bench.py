@@ -148,17 +148,20 @@ def measure(name, steps, warmup, torch, sustained_seconds=0.0, headline=False):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
 
-    # The decode step is one ~35 us call: also time it replayed from a HIP graph (one graph = one call per weight
-    # copy), which takes the host's launch path out of the measurement.
+    # The decode step is one ~35 us call: also time it replayed from a HIP graph, which takes the host's launch path out
+    # of the measurement.  One graph = four passes over the weight copies, 24 calls: a serving loop's graph holds a whole
+    # decode step of many such calls, and the few microseconds between two replays are shared by all of them.
     graph_ms = None
     if name == "decode":
+        per_graph = 4 * len(copies)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            for a in copies:
-                ops._gmm_fwd(x, a, gs, **hp, trans_rhs=False)
+            for _ in range(4):
+                for a in copies:
+                    ops._gmm_fwd(x, a, gs, **hp, trans_rhs=False)
         for _ in range(3):
             graph.replay()
-        graph_ms = _event_ms(graph.replay, max(steps // len(copies), 4), torch) / len(copies)
+        graph_ms = _event_ms(graph.replay, max(steps // per_graph, 4), torch) / per_graph
 
     # per-product launch durations, for the roofline of the dominant kernel
     if len(parts) == 1:  # the step is that one product: the timed region already is its launch duration
