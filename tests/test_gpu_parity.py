@@ -683,6 +683,85 @@ def test_stream_read_probe():
 
 
 # ---------------------------------------------------------------------------------------------------------------------
+# every launch of a call goes to the caller's stream
+# ---------------------------------------------------------------------------------------------------------------------
+
+def test_calls_on_a_side_stream_wait_for_that_stream_only():
+    """The inputs of each call are produced on a non-blocking side stream behind a long-running kernel, and the call is
+    issued on that stream at once.  A launch of the library that went to another stream (a scheduling-map kernel, a
+    finishing kernel, a zero fill) would run before its inputs exist and give a wrong result.  Covers the tile kernels
+    with the interleaved block order and the K-split, tgmm with the group order, both streaming kernels of the default
+    plan, and float32."""
+    from gpu_ragged_dot_amd import ops
+    print("side stream", flush=True)
+    hp = dict(block_m=64, block_k=64, block_n=64, interpret=False, compute_dtype=None, acc_dtype=torch.float32, chunk_m=512)
+    rng = np.random.default_rng(31)
+    side = torch.cuda.Stream()
+
+    def run(fn, host_inputs, dtype=torch.bfloat16):
+        """fn(*device tensors) on the side stream; the device tensors start as zeros and are filled on that stream."""
+        pinned = [torch.from_numpy(np.ascontiguousarray(a)).pin_memory() for a in host_inputs]
+        devs = [torch.zeros(p.shape, dtype=(torch.int32 if p.dtype == torch.int32 else dtype), device="cuda") for p in pinned]
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            torch.cuda._sleep(20_000_000)           # at least several milliseconds during which nothing of this call may start
+            for dvc, p in zip(devs, pinned):
+                dvc.copy_(p.to(dvc.dtype) if p.dtype != torch.int32 else p, non_blocking=True)
+            out = fn(*devs)
+        side.synchronize()
+        return util.to_np(out)
+
+    # tile kernels: several rounds of tiles, long and short groups (interleaved block order)
+    lens = list(rng.integers(1, 120, size=40)) + [0, 0, 700, 1300, 257, 530]
+    rng.shuffle(lens)
+    gs = np.array(lens, np.int32)
+    m, k, n, g = int(gs.sum()) + 100, 72, 4096, len(lens)
+    x = oracle.round_to(rng.standard_normal((m, k)).astype(np.float32), "bfloat16")
+    w = oracle.round_to((rng.standard_normal((g, k, n)) / k ** 0.5).astype(np.float32), "bfloat16")
+    got = run(lambda a, b, c: ops._gmm_fwd(a, b, c, **hp, trans_rhs=False), (x, w, gs))
+    util.assert_close_rows(got, oracle.gmm(x, w, gs), int(gs.sum()), util.BF16_EPS, "side stream gmm")
+    assert not np.any(got[int(gs.sum()):])
+
+    # K-split of the last round (few tiles, long contraction), trans_rhs
+    m, k, n, g = 900, 520, 7168, 5
+    lhs, rhs, dout, gs, target_m = util.make_case(3, m, k, n, g, 0.9, True, scale_rhs=True)
+    plan = _capi.Plan([v.id for v in _capi.variants() if v.name.decode() == "p256x256x32_w2x4_s4"][0], 2, 0, 2, 4)
+    got = run(lambda a, b, c: ops._gmm_fwd(a, b, c, **hp, trans_rhs=True, plan=plan), (dout, rhs, gs))
+    util.assert_close_rows(got, oracle.gmm(dout, rhs, gs, trans_rhs=True), target_m, util.BF16_EPS, "side stream dlhs")
+
+    # tgmm with the groups visited by size class
+    lens = [0, 1, 31, 64, 65, 128, 129, 300, 0, 7, 1100, 5, 40, 200, 95, 2]
+    gs = np.array(lens, np.int32)
+    m, k, n = int(gs.sum()) + 9, 264, 520
+    x = oracle.round_to(rng.standard_normal((m, k)).astype(np.float32), "bfloat16")
+    d = oracle.round_to(rng.standard_normal((m, n)).astype(np.float32), "bfloat16")
+    plan = _capi.Plan(-1, 0, 0, 1)
+    got = run(lambda a, b, c: ops._tgmm_fwd(a, b, c, **hp, plan=plan), (x, d, gs))
+    util.assert_close_groups(got, oracle.tgmm(x, d, gs), gs != 0, util.TGMM_BF16_EPS, "side stream tgmm")
+    assert not np.any(got[gs == 0])
+
+    # the streaming kernels of the default plan: whole-row slices + finishing kernel, and the trans_rhs form
+    m, k, n, g = 48, 1024, 512, 64
+    lhs, rhs, _, gs, target_m = util.make_case(5, m, k, n, g, 0.9, True, scale_rhs=True)
+    assert _capi.default_plan(_capi.OP_GMM, m, k, n, g).decode_nb == _capi.RD_DECODE_ROWS
+    got = run(lambda a, b, c: ops._gmm_fwd(a, b, c, **hp, trans_rhs=False), (lhs, rhs, gs))
+    util.assert_close_rows(got, oracle.gmm(lhs, rhs, gs), target_m, util.BF16_EPS, "side stream rows")
+    assert not np.any(got[target_m:])
+    rhs_t = np.ascontiguousarray(rhs.transpose(0, 2, 1))
+    got = run(lambda a, b, c: ops._gmm_fwd(a, b, c, **hp, trans_rhs=True), (lhs, rhs_t, gs))
+    util.assert_close_rows(got, oracle.gmm(lhs, rhs, gs), target_m, util.BF16_EPS, "side stream rows, weights transposed")
+
+    # float32
+    m, k, n, g = 300, 130, 77, 6
+    rng2 = np.random.default_rng(8)
+    x = rng2.standard_normal((m, k)).astype(np.float32)
+    w = (rng2.standard_normal((g, k, n)) / k ** 0.5).astype(np.float32)
+    gs = oracle.generate_group_sizes(4, g, 260)
+    got = run(lambda a, b, c: ops._gmm_fwd(a, b, c, **hp, trans_rhs=False), (x, w, gs), dtype=torch.float32)
+    util.assert_close_rows(got, oracle.gmm(x, w, gs, out_dtype="float32"), 260, 5e-4, "side stream float32")
+
+
+# ---------------------------------------------------------------------------------------------------------------------
 # HIP graph capture: no entry point reads device data on the host, so a captured step replays correctly
 # ---------------------------------------------------------------------------------------------------------------------
 
