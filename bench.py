@@ -403,6 +403,33 @@ def schedule_context(torch):
             fn()
         out[label] = _event_ms(fn, 20, torch)
     out["plans"] = {"dlhs": _plan_text(plan, planner), "drhs": _plan_text(tuned, planner)}
+
+    # The workload taken apart: the same launches with only the groups of up to 256 rows, only the longer ones (the
+    # others' sizes set to zero; the rows in use are then the first sum(group_sizes) ones - timing only), and for drhs
+    # with every group empty (its 7.5 GB of stores and nothing else) beside a plain zero fill of the same tensor.
+    # A launch takes about the sum of its two kinds of tiles, not their maximum.
+    sizes = gs.cpu()
+    short = torch.where(sizes <= 256, sizes, torch.zeros_like(sizes)).cuda()
+    long_ = torch.where(sizes > 256, sizes, torch.zeros_like(sizes)).cuda()
+    none = torch.zeros_like(gs)
+    parts = {}
+    for label, sel in (("all", gs), ("groups_up_to_256_rows", short), ("groups_over_256_rows", long_), ("no_rows", none)):
+        fns = {"fwd": lambda: ops._gmm_fwd(x, A, sel, **HP, acc_dtype=torch.float32, trans_rhs=False),
+               "dlhs": lambda: ops._gmm_fwd(dout, A, sel, **HP, acc_dtype=torch.float32, trans_rhs=True),
+               "drhs": lambda: ops._tgmm_fwd(x, dout, sel, **HP, acc_dtype=torch.float32)}
+        row = {"rows": int(sel.sum().item()), "groups": int((sel > 0).sum().item())}
+        for key, fn in fns.items():
+            if label == "no_rows" and key != "drhs":
+                continue
+            for _ in range(10):   # (the first launches after a pause run at a lower clock)
+                fn()
+            row[key] = _event_ms(fn, 10, torch)
+        parts[label] = row
+    dA = torch.empty((g, k, n), dtype=torch.bfloat16, device="cuda")
+    for _ in range(3):
+        dA.zero_()
+    parts["zero_fill_of_the_drhs_result"] = _event_ms(lambda: dA.zero_(), 10, torch)
+    out["taken_apart"] = parts
     return out
 
 
