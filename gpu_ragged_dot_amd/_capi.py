@@ -21,6 +21,7 @@ RD_DTYPE_BF16 = 0
 RD_DTYPE_F32 = 1
 RD_DTYPE_F32_BF16 = 2  # float32 arrays rounded to bfloat16 for the bf16 matrix cores (compute_dtype=bfloat16)
 RD_DTYPE_F8E4M3_BF16 = 3  # float8 e4m3fn operands widened to bfloat16 for the bf16 matrix cores, bfloat16 out
+RD_DTYPE_F16 = 4  # float16 arrays on the float16 matrix-core instruction, fp32 accumulation, float16 out
 
 RD_OK = 0
 RD_ERR_INVALID_ARGUMENT = -1

@@ -15,6 +15,8 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 typedef uint16_t bf16_bits;  // storage type of a bf16 element in HBM / LDS
+typedef _Float16 f16_t;      // a float16 (IEEE half) element; in LDS its 16 bits travel as bf16_bits
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 
 // fp32 -> bf16, round to nearest even (v_cvt_pk_bf16_f32 on gfx950).
 __device__ __forceinline__ bf16_bits f32_to_bf16(float f) {
@@ -24,6 +26,27 @@ __device__ __forceinline__ bf16_bits f32_to_bf16(float f) {
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+
+// fp32 -> float16, round to nearest even (v_cvt_f16_f32), and two of them in one word
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+  const f16_t l = (f16_t)lo, h = (f16_t)hi;
+  return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
+}
+// two accumulator values as two 16-bit output elements: float16 (HALF) or bf16
+template <bool HALF>
+__device__ __forceinline__ uint32_t pack_out_x2(float lo, float hi) {
+  if constexpr (HALF) return pack_f16x2(lo, hi);
+  else return pack_bf16x2(lo, hi);
+}
+// One 32x32x16 matrix-core instruction on 16-bit operands: 8 contraction-consecutive elements per lane and operand, as
+// bf16 or (HALF) as float16 - the same bits in the same places, another instruction.
+template <bool HALF>
+__device__ __forceinline__ f32x16_t mfma_32x32x16(bf16x8_t a, bf16x8_t b, f32x16_t c) {
+  if constexpr (HALF)
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
 
 typedef uint8_t fp8_bits;  // storage type of an OCP float8 e4m3fn element in HBM

@@ -17,10 +17,10 @@ namespace rd {
 
 // B_AUX: cache policy of the B operand's loads (0 = default, kCachePolicyStream = read once, do not keep in L2).
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, bool A_KMAJOR_, bool B_KMAJOR_, int STAGES_,
-          bool PINGPONG_ = false, int B_AUX_ = 0>
+          bool PINGPONG_ = false, int B_AUX_ = 0, bool HALF_ = false>
 struct DldsCfg {
-  typedef bf16_bits Elem;
-  static constexpr bool F32 = false;
+  typedef bf16_bits Elem;  // 16 bits per element: bf16, or float16 with HALF (same data movement, another instruction)
+  static constexpr bool F32 = false, HALF = HALF_;
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
   static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = true, DLDS = true, PINGPONG = PINGPONG_, MIXED = false,
                         SPLITK = true;
@@ -263,8 +263,8 @@ __device__ __forceinline__ void store_accumulators(const f32x16_t (&acc)[C::TM][
         const int row = i * 32 + (lane & 31);
         const int col = j * 32 + 8 * g + 4 * (lane >> 5);
         u32x2_t w;
-        w[0] = pack_bf16x2(acc[i][j][4 * g + 0], acc[i][j][4 * g + 1]);
-        w[1] = pack_bf16x2(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+        w[0] = pack_out_x2<C::HALF>(acc[i][j][4 * g + 0], acc[i][j][4 * g + 1]);
+        w[1] = pack_out_x2<C::HALF>(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
         *reinterpret_cast<u32x2_t*>(st + row * C::EPI_PITCH + col * 2) = w;
       }
   constexpr int CPR = C::WN / 8;        // 16-byte chunks per patch row
@@ -395,7 +395,7 @@ __device__ __forceinline__ void gemm_tile_dlds(const bf16_bits* __restrict__ Ap,
         for (int i = 0; i < C::TM; ++i)
 #pragma unroll
           for (int j = 0; j < C::TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
+            acc[i][j] = mfma_32x32x16<C::HALF>(fb[cur][j], fa[cur][i], acc[i][j]);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -506,7 +506,7 @@ __device__ __forceinline__ void gemm_tile_pingpong(const bf16_bits* __restrict__
         for (int i = 0; i < C::TM; ++i)
 #pragma unroll
           for (int j = 0; j < C::TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
+            acc[i][j] = mfma_32x32x16<C::HALF>(fb[ks][j], fa[ks][i], acc[i][j]);
     }
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);

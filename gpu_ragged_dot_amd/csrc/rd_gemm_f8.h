@@ -24,7 +24,7 @@ template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int STAGES_, int BK_ = 6
 struct F8Cfg {
   typedef fp8_bits Elem;
   typedef bf16_bits Out;
-  static constexpr bool F32 = false, F8DIRECT = true;
+  static constexpr bool F32 = false, F8DIRECT = true, HALF = false;
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
   static constexpr int B_AUX = B_AUX_;
   static_assert(BK == 64 || BK == 128, "contraction slab");

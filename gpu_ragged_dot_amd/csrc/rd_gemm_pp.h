@@ -12,7 +12,7 @@ template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, bool A_KMAJOR_, bool B_K
           int B_S_>
 struct PpCfg {
   typedef bf16_bits Elem;
-  static constexpr bool F32 = false;
+  static constexpr bool F32 = false, HALF = false;
   static constexpr int BM = BM_, BN = BN_, BK = 32, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
   static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = true, DLDS = true, PINGPONG = true, MIXED = true,
                         SPLITK = true;
@@ -191,7 +191,7 @@ __device__ __forceinline__ void gemm_tile_pingpong_mixed(const bf16_bits* __rest
         for (int i = 0; i < C::TM; ++i)
 #pragma unroll
           for (int j = 0; j < C::TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
+            acc[i][j] = mfma_32x32x16<C::HALF>(fb[ks][j], fa[ks][i], acc[i][j]);
     }
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);

@@ -23,12 +23,15 @@ namespace rd {
 // accumulation and stored as float32 - the reference's compute_dtype = bfloat16 on float32 arrays
 // (gpu_ragged_dot.py:116-119, 145, 149).  fp8_bits: float8 e4m3fn operands, widened (exactly) to bf16 on their way into
 // LDS, bf16 matrix cores with fp32 accumulation, bf16 out.
+// f16_t: float16 arrays on the float16 matrix-core instruction (v_mfma_f32_32x32x16_f16), fp32 accumulation, float16 out
+// (rounded to nearest even); the 16-bit patterns move through the stager and LDS exactly as bf16 ones do.
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, bool A_KMAJOR_, bool B_KMAJOR_, bool VEC_,
           typename Src = bf16_bits>
 struct TileCfg {
   typedef Src Elem;
   typedef typename std::conditional<sizeof(Src) == 1, bf16_bits, Src>::type Out;  // element type of the output
   static constexpr bool F32 = false;
+  static constexpr bool HALF = std::is_same<Src, f16_t>::value;  // float16 operands and matrix-core instruction
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
   static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = VEC_, DLDS = false, PINGPONG = false, MIXED = false,
                         SPLITK = false;
@@ -80,7 +83,8 @@ struct OperandStager {
     }
   }
   static __device__ __forceinline__ bf16_bits elem(const Src* p) {
-    if constexpr (sizeof(Src) == 2) return *p;
+    if constexpr (std::is_same<Src, f16_t>::value) return __builtin_bit_cast(bf16_bits, *p);
+    else if constexpr (sizeof(Src) == 2) return *p;
     else if constexpr (sizeof(Src) == 1) return (bf16_bits)fp8e4m3_to_bf16(*p);
     else return f32_to_bf16(*p);
   }
@@ -215,7 +219,11 @@ __device__ __forceinline__ void gemm_tile(const typename C::Elem* __restrict__ A
       for (int i = 0; i < C::TM; ++i)
 #pragma unroll
         for (int j = 0; j < C::TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+          if constexpr (C::HALF)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, fa[i]), __builtin_bit_cast(f16x8_t, fb[j]),
+                                                              acc[i][j], 0, 0, 0);
+          else
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
     }
     if (more) {
       sa.store(ra, nxt);
@@ -234,7 +242,8 @@ __device__ __forceinline__ void gemm_tile(const typename C::Elem* __restrict__ A
       for (int v = 0; v < 16; ++v) {
         const int row = wm * C::WM + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
         if (row < a_lim && col < b_lim) {
-          if constexpr (sizeof(typename C::Out) == 2) Op[(size_t)row * ldo + col] = f32_to_bf16(acc[i][j][v]);
+          if constexpr (C::HALF) Op[(size_t)row * ldo + col] = (f16_t)acc[i][j][v];
+          else if constexpr (sizeof(typename C::Out) == 2) Op[(size_t)row * ldo + col] = f32_to_bf16(acc[i][j][v]);
           else Op[(size_t)row * ldo + col] = acc[i][j][v];
         }
       }

@@ -15,10 +15,10 @@
 
 namespace rd {
 
-template <int BM_, int BN_, bool A_KMAJOR_, bool B_KMAJOR_, int STAGES_>
+template <int BM_, int BN_, bool A_KMAJOR_, bool B_KMAJOR_, int STAGES_, bool HALF_ = false>
 struct W4Cfg {
-  typedef bf16_bits Elem;
-  static constexpr bool F32 = false, W4 = true;
+  typedef bf16_bits Elem;  // 16 bits per element: bf16, or float16 with HALF
+  static constexpr bool F32 = false, W4 = true, HALF = HALF_;
   static constexpr int BM = BM_, BN = BN_, BK = 32, WAVES_M = 2, WAVES_N = 2, STAGES = STAGES_;
   static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, VEC = true, DLDS = true, PINGPONG = false, MIXED = false,
                         SPLITK = true;
@@ -128,7 +128,7 @@ __device__ __forceinline__ void w4_kloop(const bf16_bits* __restrict__ Ap, int l
       }
       constexpr int T0 = MF - 2 * LdB::PER;
       if (t >= T0 && ((t - T0) & 1) == 0 && more_b) issue_one_b(kt + S - 1, prev_off, (t - T0) >> 1, steady_tag);
-      if (LIVE) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[0][j], fa[0][i], acc[i][j], 0, 0, 0);
+      if (LIVE) acc[i][j] = mfma_32x32x16<C::HALF>(fb[0][j], fa[0][i], acc[i][j]);
       __builtin_amdgcn_sched_barrier(0);
     }
     if (more_b) lb.advance();
@@ -152,7 +152,7 @@ __device__ __forceinline__ void w4_kloop(const bf16_bits* __restrict__ Ap, int l
       }
       constexpr int T0 = MF - 2 * LdA::PER;
       if (t >= T0 && ((t - T0) & 1) == 0 && more_a) issue_one_a(kt + S, cur, (t - T0) >> 1, steady_tag);
-      if (LIVE) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[1][j], fa[1][i], acc[i][j], 0, 0, 0);
+      if (LIVE) acc[i][j] = mfma_32x32x16<C::HALF>(fb[1][j], fa[1][i], acc[i][j]);
       __builtin_amdgcn_sched_barrier(0);
     }
     if (more_a) la.advance();

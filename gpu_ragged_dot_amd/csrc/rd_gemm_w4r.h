@@ -22,10 +22,10 @@
 
 namespace rd {
 
-template <int BM_, int BN_>
+template <int BM_, int BN_, bool HALF_ = false>
 struct W4RCfg {
-  typedef bf16_bits Elem;
-  static constexpr bool F32 = false, W4 = true, W4R = true;
+  typedef bf16_bits Elem;  // 16 bits per element: bf16, or float16 with HALF
+  static constexpr bool F32 = false, W4 = true, W4R = true, HALF = HALF_;
   static constexpr int BM = BM_, BN = BN_, BK = 64, WAVES_M = 2, WAVES_N = 2, STAGES = 2;
   static constexpr bool A_KMAJOR = true, B_KMAJOR = true, VEC = true, DLDS = true, PINGPONG = false, MIXED = false, SPLITK = true;
   static constexpr int NW = 4, NT = 256;
@@ -167,7 +167,7 @@ __device__ __forceinline__ void w4r_kloop(const bf16_bits* __restrict__ Ap, int 
           if (((m - R0) & 1) == 0) { if (write_next) commit_one(next_tag, next_off, q); }
           else if (fetch_far) fetch_one(next_tag, t + 3, q, steady_tag);
         }
-        if (LIVE) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[u & 1][j], fa[u & 1][i], acc[i][j], 0, 0, 0);
+        if (LIVE) acc[i][j] = mfma_32x32x16<C::HALF>(fb[u & 1][j], fa[u & 1][i], acc[i][j]);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -193,7 +193,7 @@ __device__ __forceinline__ void w4r_kloop(const bf16_bits* __restrict__ Ap, int 
         if (((m - R0) & 1) == 0) { if (write_after) commit_one(w4r_detail::Int<1 - NEXT>{}, cur_off, q); }
         else if (fetch_after) fetch_one(w4r_detail::Int<1 - NEXT>{}, t + 4, q, steady_tag);
       }
-      if (LIVE) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[1][j], fa[1][i], acc[i][j], 0, 0, 0);
+      if (LIVE) acc[i][j] = mfma_32x32x16<C::HALF>(fb[1][j], fa[1][i], acc[i][j]);
       __builtin_amdgcn_sched_barrier(0);
     }
   };

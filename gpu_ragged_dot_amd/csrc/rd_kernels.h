@@ -87,7 +87,7 @@ __device__ __forceinline__ void run_tile(const typename C::Elem* Ap, int lda, in
     // The register-staged form has four 64-wide slabs to fill before it runs and pays for that on a short contraction:
     // below kW4RMinK the 32-wide direct-to-LDS form of the same core takes the tile.
     if (klen >= kW4RMinK) gemm_tile_w4r<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
-    else gemm_tile_w4<W4Cfg<C::BM, C::BN, true, true, 5>>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
+    else gemm_tile_w4<W4Cfg<C::BM, C::BN, true, true, 5, C::HALF>>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
   }
   else if constexpr (IsW4<C>::value) gemm_tile_w4<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
   else if constexpr (C::MIXED) gemm_tile_pingpong_mixed<C>(Ap, lda, a_lim, Bp, ldb, b_lim, klen, Op, ldo, smem, sk);
@@ -110,7 +110,7 @@ template <class C, int ROWS>
 struct ShortTileCfg {
   static constexpr int BK = C::B_KMAJOR ? 64 : 32;
   static constexpr int STAGES = (160 * 1024) / ((ROWS + C::BN) * BK * 2);
-  typedef DldsCfg<ROWS, C::BN, BK, 1, 4, true, C::B_KMAJOR, STAGES, false, kCachePolicyStream> type;
+  typedef DldsCfg<ROWS, C::BN, BK, 1, 4, true, C::B_KMAJOR, STAGES, false, kCachePolicyStream, C::HALF> type;
 };
 
 // How the last round of a gmm launch is cut along K.  The device runs num_cus tiles at a time; when the live tiles do

@@ -1,6 +1,6 @@
 // One compiled tile shape.  Built once per entry of the variant list in the Makefile, with
 //   -DRD_BM= -DRD_BN= -DRD_BK= -DRD_WAVES_M= -DRD_WAVES_N= -DRD_VEC= -DRD_NAME= [-DRD_DLDS=1|2|3 -DRD_STAGES= -DRD_PINGPONG=1
-//   -DRD_F32=1|2|3]
+//   -DRD_F32=1|2|3|4]
 // and exports a getter rd_variant_<name>() for its TileVariant record that the C-ABI file collects.
 #include "rd_kernels.h"
 
@@ -24,7 +24,12 @@
 #endif
 
 namespace rd {
-#if RD_F32 == 3 && RD_DLDS
+#if RD_F32 == 4 && RD_DLDS == 3
+// float16 arrays on the four-wave direct-to-LDS core: the bf16 core's data movement with the float16 instruction
+typedef W4Cfg<RD_BM, RD_BN, /*A K-major*/ true, /*B K-major*/ false, RD_STAGES, true> CfgNN;
+typedef W4RCfg<RD_BM, RD_BN, true> CfgNT;
+typedef W4Cfg<RD_BM, RD_BN, false, false, RD_STAGES, true> CfgTN;
+#elif RD_F32 == 3 && RD_DLDS
 // float8 e4m3fn arrays on the float8 matrix-core instruction, direct-to-LDS (rd_gemm_f8.h).  tgmm reads x^T as an
 // MN-major operand, whose slab rows span the tile's rows: only for tile heights that are multiples of 256.
 typedef F8Cfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, RD_STAGES, 64, 0, /*A K-major*/ true, /*B K-major*/ false, RD_PINGPONG != 0> CfgNN;
@@ -39,6 +44,11 @@ typedef F8Cfg<RD_BM, RD_BN, RD_WAVES_M, RD_WAVES_N, RD_STAGES, 64, 0, false, fal
 typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, /*A K-major*/ true, /*B K-major*/ false, RD_VEC != 0, fp8_bits> CfgNN;
 typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, true, true, RD_VEC != 0, fp8_bits> CfgNT;
 typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, false, false, RD_VEC != 0, fp8_bits> CfgTN;
+#elif RD_F32 == 4
+// float16 arrays on the float16 matrix-core instruction, float16 out
+typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, /*A K-major*/ true, /*B K-major*/ false, RD_VEC != 0, f16_t> CfgNN;
+typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, true, true, RD_VEC != 0, f16_t> CfgNT;
+typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, false, false, RD_VEC != 0, f16_t> CfgTN;
 #elif RD_F32 == 2
 // float32 arrays, rounded to bf16 on the way into LDS, bf16 matrix cores, float32 out (compute_dtype = bfloat16)
 typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, /*A K-major*/ true, /*B K-major*/ false, RD_VEC != 0, float> CfgNN;
@@ -74,7 +84,7 @@ typedef TileCfg<RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, false, false, RD_VE
 extern "C" const rd::TileVariant* RD_CAT(rd_variant_, RD_NAME)() {
   static const rd::TileVariant v = {
       RD_STR(RD_NAME), RD_BM, RD_BN, RD_BK, RD_WAVES_M, RD_WAVES_N, RD_VEC, /*dtype: RD_DTYPE_* */ RD_F32, RD_DLDS != 0, RD_STAGES,
-      /*splitk*/ RD_DLDS != 0 && (!RD_F32 || RD_F32 == 3),
+      /*splitk*/ RD_DLDS != 0 && (!RD_F32 || RD_F32 == 3 || RD_F32 == 4),
 #ifdef RD_NO_TGMM
       &rd::launch_gmm<rd::CfgNN, false>, &rd::launch_gmm<rd::CfgNT, true>, nullptr};
 #else

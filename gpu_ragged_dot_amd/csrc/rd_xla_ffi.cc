@@ -27,6 +27,7 @@ int dtype_code(ffi::DataType t, bool compute_bf16) {
   if (t == ffi::DataType::BF16) return RD_DTYPE_BF16;
   if (t == ffi::DataType::F32) return compute_bf16 ? RD_DTYPE_F32_BF16 : RD_DTYPE_F32;
   if (t == ffi::DataType::F8E4M3FN) return RD_DTYPE_F8E4M3_BF16;  // the result buffer is then bfloat16
+  if (t == ffi::DataType::F16) return RD_DTYPE_F16;
   return -1;
 }
 

@@ -52,6 +52,8 @@ def _dtype_code(dtype, compute_dtype, acc_dtype) -> int:
     compute = dtype if compute_dtype is None else jnp.dtype(compute_dtype)
     if dtype == jnp.bfloat16 and compute in (jnp.dtype(jnp.bfloat16), jnp.dtype(jnp.float32)):
         return _capi.RD_DTYPE_BF16  # widening bf16 operands changes nothing: exact products, fp32 accumulation
+    if dtype == jnp.float16 and compute in (jnp.dtype(jnp.float16), jnp.dtype(jnp.float32)):
+        return _capi.RD_DTYPE_F16  # as for bfloat16: products of float16 values are exact in fp32
     if dtype == jnp.float32 and compute == jnp.dtype(jnp.float32):
         return _capi.RD_DTYPE_F32
     if dtype == jnp.float32 and compute == jnp.dtype(jnp.bfloat16):

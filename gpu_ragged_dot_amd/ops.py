@@ -18,7 +18,7 @@ from .planner import CHUNK_M, DEFAULT_BLOCK_K, DEFAULT_BLOCK_M, DEFAULT_BLOCK_N
 __all__ = ["gmm", "tgmm", "ragged_dot", "trans_ragged_dot", "ragged_dot_vjp", "make_group_metadata"]
 
 _DTYPES = {torch.bfloat16: _capi.RD_DTYPE_BF16, torch.float32: _capi.RD_DTYPE_F32,
-           torch.float8_e4m3fn: _capi.RD_DTYPE_F8E4M3_BF16}
+           torch.float8_e4m3fn: _capi.RD_DTYPE_F8E4M3_BF16, torch.float16: _capi.RD_DTYPE_F16}
 
 
 def _out_dtype(t: torch.Tensor) -> torch.dtype:
@@ -31,7 +31,7 @@ def _dtype_code(t: torch.Tensor, compute_dtype, acc_dtype) -> int:
     """Element-type code for the C ABI from the storage dtype and the reference's ``compute_dtype``
     (gpu_ragged_dot.py:116-119, 145: operands are cast to compute_dtype before the dot; None = the storage dtype)."""
     if t.dtype not in _DTYPES:
-        raise TypeError(f"unsupported dtype {t.dtype}; operands are bfloat16, float32 or float8_e4m3fn")
+        raise TypeError(f"unsupported dtype {t.dtype}; operands are bfloat16, float16, float32 or float8_e4m3fn")
     if acc_dtype not in (None, torch.float32):
         raise NotImplementedError("accumulation is always float32 on the matrix cores")
     if t.dtype == torch.float8_e4m3fn:
@@ -42,6 +42,8 @@ def _dtype_code(t: torch.Tensor, compute_dtype, acc_dtype) -> int:
         return _DTYPES[t.dtype]
     if t.dtype == torch.float32 and compute_dtype == torch.bfloat16:
         return _capi.RD_DTYPE_F32_BF16  # rounded to bf16 on the way to the bf16 matrix cores, float32 out
+    if t.dtype == torch.float16 and compute_dtype == torch.float32:
+        return _capi.RD_DTYPE_F16  # as for bfloat16 below: products of float16 values are exact in fp32
     if t.dtype == torch.bfloat16 and compute_dtype == torch.float32:
         # widening bf16 operands changes nothing: their products are exact in fp32 and accumulation is fp32 anyway
         return _capi.RD_DTYPE_BF16

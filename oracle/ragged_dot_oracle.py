@@ -90,11 +90,14 @@ def f32_to_float8_e4m3fn(a: np.ndarray) -> np.ndarray:
 
 
 def round_to(a: np.ndarray, dtype: str) -> np.ndarray:
-    """Round a float array to ``dtype`` ('bfloat16' | 'float32') and return it as float32 values."""
+    """Round a float array to ``dtype`` ('bfloat16' | 'float16' | 'float32') and return it as float32 values."""
     if dtype == "bfloat16":
         return bf16_bits_to_f32(f32_to_bf16_bits(a)).reshape(np.shape(a))
     if dtype == "float32":
         return np.asarray(a, dtype=np.float32)
+    if dtype == "float16":  # IEEE half, round to nearest even (numpy's own conversion)
+        with np.errstate(over="ignore"):  # beyond 65504 the result is infinity, as the format defines
+            return np.asarray(a, dtype=np.float32).astype(np.float16).astype(np.float32)
     raise ValueError(f"unsupported dtype {dtype!r}")
 
 

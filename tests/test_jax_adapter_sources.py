@@ -138,17 +138,17 @@ def test_result_element_type_rule_matches_the_python_side():
         shim = f.read()
     # element types the shim accepts
     known = re.findall(r"t == ffi::DataType::([A-Z0-9]+)", _shim_function(shim, "dtype_code"))
-    assert sorted(known) == ["BF16", "F32", "F8E4M3FN"], known
+    assert sorted(known) == ["BF16", "F16", "F32", "F8E4M3FN"], known
     # result_type(): `if (t == ffi::DataType::X) return ffi::DataType::Y;` lines, then `return t;`
     body = _shim_function(shim, "result_type")
     special = dict(re.findall(r"if \(t == ffi::DataType::([A-Z0-9]+)\) return ffi::DataType::([A-Z0-9]+);", body))
     assert re.search(r"return t;\s*$", body.strip())
     shim_rule = {t: special.get(t, t) for t in known}
     # jax_adapter._out_dtype evaluated with stand-ins for jnp
-    names = {"BF16": "bfloat16", "F32": "float32", "F8E4M3FN": "float8_e4m3fn"}
+    names = {"BF16": "bfloat16", "F16": "float16", "F32": "float32", "F8E4M3FN": "float8_e4m3fn"}
 
     class _Jnp:
-        bfloat16, float32, float8_e4m3fn = "bfloat16", "float32", "float8_e4m3fn"
+        bfloat16, float16, float32, float8_e4m3fn = "bfloat16", "float16", "float32", "float8_e4m3fn"
         dtype = staticmethod(lambda d: d)
 
     fn = _func(_tree(), "_out_dtype")

@@ -33,6 +33,27 @@ def test_bf16_matches_torch():
     np.testing.assert_array_equal(ours, theirs)
 
 
+def test_float16_round_to_nearest_even_known_values():
+    """round_to(.., 'float16'): IEEE half, 10 mantissa bits, ties to even, overflow to infinity, subnormals down to 2^-24."""
+    r = lambda v: float(oracle.round_to(np.array([v], np.float32), "float16")[0])
+    assert r(1.0 + 2.0 ** -11) == 1.0                       # half-way between 1 and 1 + 2^-10, even mantissa below
+    assert r(1.0 + 3 * 2.0 ** -11) == 1.0 + 2.0 ** -9       # half-way, odd mantissa below: up to the even one
+    assert r(1.0 + 2.0 ** -11 + 2.0 ** -20) == 1.0 + 2.0 ** -10   # just above half-way
+    assert r(65504.0) == 65504.0 and r(65519.0) == 65504.0 and np.isinf(r(65520.0))   # largest value; the tie goes to inf
+    assert r(2.0 ** -24) == 2.0 ** -24 and r(2.0 ** -25) == 0.0 and r(1.5 * 2.0 ** -24) == 2.0 ** -23   # subnormals, ties to even
+    assert r(-0.1) == -r(0.1) and abs(r(0.1) - 0.1) <= 2.0 ** -14
+
+
+def test_float16_matches_torch():
+    import torch
+
+    a = np.random.default_rng(1).normal(size=10000).astype(np.float32) * 300
+    a[:4] = [7e4, -7e4, 1e-7, 6e-8]
+    ours = oracle.round_to(a, "float16")
+    theirs = torch.from_numpy(a).to(torch.float16).float().numpy()
+    np.testing.assert_array_equal(ours, theirs)
+
+
 # ---- scheduling map (gpu_ragged_dot.py:70-90) -------------------------------------------------------------------------
 
 def test_metadata_hand_computed():
