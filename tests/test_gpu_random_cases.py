@@ -1,9 +1,10 @@
 """Seeded random cases against the oracle: shapes (aligned and odd pitches, a few with several rounds of 256 x 256
 tiles or a long contraction), group sizes (random partitions, Zipf-like with empty groups, everything in one group,
-lengths around tile boundaries, all empty; with and without a zero tail), bf16 and float32, all three products, the
+lengths around tile boundaries, all empty; with and without a zero tail), bf16, float32 and float16, all three products, the
 default plan or a random compiled variant with a random tile walk and K-split setting, and the streaming kernels forced.
 A call the library refuses must refuse with RD_ERR_UNSUPPORTED or RD_ERR_INVALID_ARGUMENT; everything it accepts must
-match the oracle at the reference's tolerances (tests.py:127,144,168,183; float32 5e-4 / 1e-4, tests.py:93), with the
+match the oracle at the reference's tolerances (tests.py:127,144,168,183; float32 5e-4 / 1e-4, tests.py:93; float16 a
+fifth / half of the bf16 ones), with the
 tail rows and the empty groups' slices exactly zero."""
 
 import numpy as np
@@ -51,7 +52,7 @@ def _group_sizes(rng, g, m):
 def _one_case(seed, it, variants):
     rng = np.random.default_rng(seed * 100003 + it)
     op = ["gmm", "gmm_t", "tgmm"][int(rng.integers(0, 3))]
-    dt = "bfloat16" if rng.random() < 0.8 else "float32"
+    dt = ["bfloat16", "float32", "float16"][int(np.searchsorted([0.7, 0.85], rng.random(), side="right"))]
     aligned = rng.random() < 0.7
     big = rng.random() < 0.25
     m = int(rng.integers(1, 2500 if big else 600))
@@ -73,7 +74,7 @@ def _one_case(seed, it, variants):
     gs = _group_sizes(rng, g, m)
     plan, plan_txt = None, "default"
     if rng.random() < 0.6:
-        code = _capi.RD_DTYPE_BF16 if dt == "bfloat16" else _capi.RD_DTYPE_F32
+        code = {"bfloat16": _capi.RD_DTYPE_BF16, "float32": _capi.RD_DTYPE_F32, "float16": _capi.RD_DTYPE_F16}[dt]
         cand = [v for v in variants if v.dtype == code and (not v.vec or aligned)]
         v = cand[int(rng.integers(0, len(cand)))]
         gm, gn, sk = int(rng.integers(0, 9)), int(rng.integers(0, 9)), int(rng.choice([0, 0, -1, 2, 8]))
@@ -86,10 +87,10 @@ def _one_case(seed, it, variants):
     x = oracle.round_to(rng.standard_normal((m, k)).astype(np.float32), dt)
     w = oracle.round_to((rng.standard_normal((g, k, n)) / max(k, 1) ** 0.5).astype(np.float32), dt)
     d = oracle.round_to(rng.standard_normal((m, n)).astype(np.float32), dt)
-    tdt = torch.bfloat16 if dt == "bfloat16" else torch.float32
+    tdt = {"bfloat16": torch.bfloat16, "float32": torch.float32, "float16": torch.float16}[dt]
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda().to(tdt)
-    eps_rows = util.BF16_EPS if dt == "bfloat16" else 5e-4
-    eps_groups = util.TGMM_BF16_EPS if dt == "bfloat16" else 1e-4
+    eps_rows = {"bfloat16": util.BF16_EPS, "float32": 5e-4, "float16": util.BF16_EPS / 5}[dt]
+    eps_groups = {"bfloat16": util.TGMM_BF16_EPS, "float32": 1e-4, "float16": util.TGMM_BF16_EPS / 2}[dt]
     live = int(gs.sum())
     try:
         if op == "gmm":
