@@ -120,9 +120,11 @@ __global__ __launch_bounds__(64) void moe_rank_kernel(const int32_t* __restrict_
 template <class T> __device__ __forceinline__ float to_f32(T v);
 template <> __device__ __forceinline__ float to_f32<bf16_bits>(bf16_bits v) { return bf16_to_f32(v); }
 template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ float to_f32<f16_t>(f16_t v) { return (float)v; }
 template <class T> __device__ __forceinline__ T from_f32(float v);
 template <> __device__ __forceinline__ bf16_bits from_f32<bf16_bits>(float v) { return f32_to_bf16(v); }
 template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ f16_t from_f32<f16_t>(float v) { return (f16_t)v; }
 
 constexpr int kRowThreads = 256;
 
@@ -304,10 +306,11 @@ static int dispatch_t(hipStream_t s, const void* h, const int32_t* row_of_slot, 
 }
 
 int launch_moe_dispatch(hipStream_t s, const void* h, const int32_t* row_of_slot, const int32_t* slot_of_row,
-                        const float* row_scale, void* x, int tokens, int top_k, int d, bool f32) {
+                        const float* row_scale, void* x, int tokens, int top_k, int d, int elem) {
   if (tokens <= 0 || d <= 0) return hipSuccess;
-  return f32 ? dispatch_t<float>(s, h, row_of_slot, slot_of_row, row_scale, x, tokens, top_k, d)
-             : dispatch_t<bf16_bits>(s, h, row_of_slot, slot_of_row, row_scale, x, tokens, top_k, d);
+  return elem == 1 ? dispatch_t<float>(s, h, row_of_slot, slot_of_row, row_scale, x, tokens, top_k, d)
+       : elem == 2 ? dispatch_t<f16_t>(s, h, row_of_slot, slot_of_row, row_scale, x, tokens, top_k, d)
+                   : dispatch_t<bf16_bits>(s, h, row_of_slot, slot_of_row, row_scale, x, tokens, top_k, d);
 }
 
 template <class T>
@@ -320,16 +323,18 @@ static int combine_t(hipStream_t s, const void* y, const int32_t* row_of_slot, c
 }
 
 int launch_moe_combine(hipStream_t s, const void* y, const int32_t* row_of_slot, const float* weights, void* out,
-                       int tokens, int top_k, int d, bool f32) {
+                       int tokens, int top_k, int d, int elem) {
   if (tokens <= 0 || d <= 0) return hipSuccess;
-  return f32 ? combine_t<float>(s, y, row_of_slot, weights, out, tokens, top_k, d)
-             : combine_t<bf16_bits>(s, y, row_of_slot, weights, out, tokens, top_k, d);
+  return elem == 1 ? combine_t<float>(s, y, row_of_slot, weights, out, tokens, top_k, d)
+       : elem == 2 ? combine_t<f16_t>(s, y, row_of_slot, weights, out, tokens, top_k, d)
+                   : combine_t<bf16_bits>(s, y, row_of_slot, weights, out, tokens, top_k, d);
 }
 
 int launch_moe_combine_wgrad(hipStream_t s, const void* y, const void* dout, const int32_t* row_of_slot, float* dw,
-                             int tokens, int top_k, int d, bool f32) {
+                             int tokens, int top_k, int d, int elem) {
   if (tokens <= 0 || top_k <= 0) return hipSuccess;
-  if (f32) hipLaunchKernelGGL(moe_combine_wgrad_kernel<float>, dim3(tokens), dim3(kRowThreads), 0, s, (const float*)y, (const float*)dout, row_of_slot, dw, top_k, d);
+  if (elem == 2) hipLaunchKernelGGL(moe_combine_wgrad_kernel<f16_t>, dim3(tokens), dim3(kRowThreads), 0, s, (const f16_t*)y, (const f16_t*)dout, row_of_slot, dw, top_k, d);
+  else if (elem == 1) hipLaunchKernelGGL(moe_combine_wgrad_kernel<float>, dim3(tokens), dim3(kRowThreads), 0, s, (const float*)y, (const float*)dout, row_of_slot, dw, top_k, d);
   else hipLaunchKernelGGL(moe_combine_wgrad_kernel<bf16_bits>, dim3(tokens), dim3(kRowThreads), 0, s, (const bf16_bits*)y, (const bf16_bits*)dout, row_of_slot, dw, top_k, d);
   return (int)hipGetLastError();
 }

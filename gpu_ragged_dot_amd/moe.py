@@ -55,8 +55,8 @@ def route(expert_ids: torch.Tensor, num_groups: int) -> Routing:
 
 
 def _dtype(t: torch.Tensor) -> int:
-    if t.dtype not in _DTYPES:
-        raise TypeError(f"unsupported dtype {t.dtype}; rows are bfloat16 or float32")
+    if t.dtype not in _DTYPES or t.dtype == torch.float8_e4m3fn:
+        raise TypeError(f"unsupported dtype {t.dtype}; rows are bfloat16, float16 or float32")
     return _DTYPES[t.dtype]
 
 

@@ -147,16 +147,17 @@ def test_route_fixture_on_gpu(i):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16], ids=["bf16", "f32", "f16"])
 @pytest.mark.parametrize("tokens,top_k,g,d", [(64, 8, 128, 2048), (300, 2, 8, 520), (77, 3, 5, 58), (1000, 4, 16, 7)])
 def test_dispatch_combine_parity(tokens, top_k, g, d, dtype):
-    """dispatch is a copy: bit-exact.  combine sums top_k products in fp32 and rounds once: within 2^-7 (bf16) or
-    1e-5 (float32) of the float64 oracle, relative to the largest output."""
+    """dispatch is a copy: bit-exact.  combine sums top_k products in fp32 and rounds once: within 2^-7 (bf16), 2^-10
+    (float16) or 1e-5 (float32) of the float64 oracle, relative to the largest output."""
     from gpu_ragged_dot_amd import moe
     print(f"dispatch/combine tokens={tokens} top_k={top_k} g={g} d={d} {dtype}", flush=True)
     rng = np.random.default_rng(tokens + d)
     ids = _random_ids(tokens, tokens, top_k, g, 0.1)
-    rnd = (lambda a: oracle.round_to(a, "bfloat16")) if dtype == torch.bfloat16 else (lambda a: a.astype(np.float32))
+    name = {torch.bfloat16: "bfloat16", torch.float32: "float32", torch.float16: "float16"}[dtype]
+    rnd = lambda a: oracle.round_to(a, name)
     h = rnd(rng.standard_normal((tokens, d)).astype(np.float32))
     y = rnd(rng.standard_normal((tokens * top_k, d)).astype(np.float32))
     w = rng.random((tokens, top_k)).astype(np.float32)
@@ -165,7 +166,7 @@ def test_dispatch_combine_parity(tokens, top_k, g, d, dtype):
     hd, yd, wd = (torch.from_numpy(a).cuda() for a in (h, y, w))
     x = moe.dispatch(hd.to(dtype), r)
     assert np.array_equal(util.to_np(x), moe_oracle.dispatch(h, sor, top_k))
-    tol = 2.0 ** -7 if dtype == torch.bfloat16 else 1e-5
+    tol = {torch.bfloat16: 2.0 ** -7, torch.float32: 1e-5, torch.float16: 2.0 ** -10}[dtype]
     for weights, wn in ((None, None), (wd, w)):
         out = util.to_np(moe.combine(yd.to(dtype), r, weights))
         ref = moe_oracle.combine(y, ros, top_k, wn)
