@@ -195,7 +195,8 @@ int rd_probe_stream_read(void* stream, const void* src, size_t bytes, size_t blo
  *     (weights NULL = 1), fp32 accumulation, rounded once.  y is [slots, d], out is [tokens, d].  With weights NULL it
  *     is the adjoint of rd_moe_dispatch.
  *   rd_moe_combine_wgrad: dw[slot] = <y[row_of_slot[slot], :], dout[token, :]> in fp32 (0 for dropped slots).
- * weights, row_scale and dw are float32 [tokens * top_k]. */
+ * weights, row_scale and dw are float32 [tokens * top_k]; the rows (h, x, y, out, dout) are RD_DTYPE_BF16, RD_DTYPE_F32
+ * or RD_DTYPE_F16. */
 size_t rd_moe_route_workspace_bytes(int tokens, int top_k, int g);
 int rd_moe_route(void* stream, const int32_t* expert_ids, int tokens, int top_k, int g, int32_t* group_sizes,
                  int32_t* row_of_slot, int32_t* slot_of_row, void* workspace, size_t workspace_bytes);
