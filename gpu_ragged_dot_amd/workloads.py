@@ -26,6 +26,12 @@ WORKLOADS = {
     "mixtral_fwd_bwd": Workload("mixtral_fwd_bwd", 16384, 4096, 14336, 8, True, "Mixtral-8x7B up-projection, forward + dlhs + drhs"),
     "deepseek_fwd_bwd": Workload("deepseek_fwd_bwd", 32768, 7168, 2048, 256, True, "DeepSeek-V3 routed experts, Zipf-skewed sizes, ~10% empty, forward + backward"),
     "decode": Workload("decode", 64, 2048, 768, 128, False, "Qwen3-30B-A3B decode, 8 tokens x top-8, forward only"),
+    # the other projections of the same layers and a prefill batch (not benchmark configurations: shapes for the tuner,
+    # `python -m gpu_ragged_dot_amd.tune --workload <name> --write`, and for `bench.py --workload <name> --only`)
+    "mixtral_down_fwd_bwd": Workload("mixtral_down_fwd_bwd", 16384, 14336, 4096, 8, True, "Mixtral-8x7B down-projection, same routing, forward + backward"),
+    "deepseek_down_fwd_bwd": Workload("deepseek_down_fwd_bwd", 32768, 2048, 7168, 256, True, "DeepSeek-V3 routed experts' down-projection, same routing, forward + backward"),
+    "qwen3_prefill_fwd_bwd": Workload("qwen3_prefill_fwd_bwd", 32768, 2048, 768, 128, True, "Qwen3-30B-A3B expert up-projection, 4096 tokens x top-8, forward + backward"),
+    "qwen3_prefill_down_fwd_bwd": Workload("qwen3_prefill_down_fwd_bwd", 32768, 768, 2048, 128, True, "Qwen3-30B-A3B expert down-projection, 4096 tokens x top-8, forward + backward"),
 }
 
 
@@ -50,10 +56,12 @@ def zipf_counts(seed: int, total: int, g: int, s: float, n_empty: int) -> np.nda
 def group_sizes(name: str) -> np.ndarray:
     if name == "tiny":
         return np.random.default_rng(0).multinomial(512, [0.25] * 4).astype(np.int32)
-    if name in ("mixtral_fwd", "mixtral_fwd_bwd"):
+    if name in ("mixtral_fwd", "mixtral_fwd_bwd", "mixtral_down_fwd_bwd"):
         return top_k_counts(1, 8192, 8, 2)
-    if name == "deepseek_fwd_bwd":
+    if name in ("deepseek_fwd_bwd", "deepseek_down_fwd_bwd"):
         return zipf_counts(2, 32768, 256, 1.1, 26)
+    if name in ("qwen3_prefill_fwd_bwd", "qwen3_prefill_down_fwd_bwd"):
+        return top_k_counts(4, 4096, 128, 8)
     if name == "decode":
         return top_k_counts(3, 8, 128, 8)
     raise KeyError(name)
