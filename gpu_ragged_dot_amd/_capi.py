@@ -57,7 +57,7 @@ class VariantInfo(ctypes.Structure):
 
 
 RD_DECODE_ROWS = -1  # Plan.decode_nb: whole-row slices
-ABI_VERSION = 2  # RD_ABI_VERSION of include/ragged_dot_hip.h this file mirrors
+ABI_VERSION = 3  # RD_ABI_VERSION of include/ragged_dot_hip.h this file mirrors
 
 
 class Plan(ctypes.Structure):

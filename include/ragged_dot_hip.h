@@ -26,7 +26,9 @@
 extern "C" {
 #endif
 
-#define RD_ABI_VERSION 2
+/* 3: RD_DTYPE_F16; rd_plan.group_n = 1 for rd_tgmm; the workspaces hold the orders the scheduling-map kernel builds
+ * (all source compatible with 2: same structs, same signatures) */
+#define RD_ABI_VERSION 3
 
 /* Element type of the operands and the output (the same, gpu_ragged_dot.py:210,324, but for float8) and what the matrix
  * cores multiply.  RD_DTYPE_F32_BF16 is compute_dtype = bfloat16 on float32 arrays (gpu_ragged_dot.py:116-119, 145, 149): the

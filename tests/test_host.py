@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(lib, name), f"{name} declared in include/ragged_dot_hip.h but not exported"
     assert sorted(_capi.EXPORTS) == names, "the ctypes binding must cover exactly what the header declares"
-    assert _capi.lib.rd_abi_version() == 2
+    assert _capi.lib.rd_abi_version() == 3
 
 
 def test_variant_table():
