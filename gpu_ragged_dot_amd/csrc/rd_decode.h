@@ -6,11 +6,12 @@
 namespace rd {
 
 struct DecodeArgs {
-  const uint16_t* x;   // [m, k] bf16
-  const uint16_t* A;   // [g, k, n] bf16
-  uint16_t* y;         // [m, n] bf16
+  const uint16_t* x;   // [m, k] bf16 (or float16, see half)
+  const uint16_t* A;   // [g, k, n]
+  uint16_t* y;         // [m, n]
   const int32_t* group_sizes;
   int m, k, n, g;
+  int half;  // 0: the 16-bit elements are bf16; 1: float16 (same layouts, another conversion and dot instruction)
 };
 
 // nb: columns per work-group (32, 64 or 128).  Needs k % 8 == 0, n % 8 == 0 and k <= kDecodeMaxK.

@@ -24,6 +24,37 @@ constexpr int kRows = 4;    // rows of x handled per pass over the weights
 constexpr int kDepth = 8;   // 16-byte weight loads kept in flight per thread (a ring of registers)
 constexpr int kStage = 8;   // activation words a thread stages per round trip
 
+// The kernels work on 16-bit elements: bf16, or float16 when HALF is set.  Same loads, same staging, same sums in fp32;
+// what differs is how the lower / upper half of a 32-bit word becomes an fp32 value, which v_dot2 instruction multiplies
+// two pairs, and how a sum is rounded to an output element.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+template <bool HALF>
+__device__ __forceinline__ float lo_f32(uint32_t w) {
+  if constexpr (HALF) return (float)__builtin_bit_cast(f16_t, (uint16_t)(w & 0xffffu));
+  else return __builtin_bit_cast(float, w << 16);
+}
+template <bool HALF>
+__device__ __forceinline__ float hi_f32(uint32_t w) {
+  if constexpr (HALF) return (float)__builtin_bit_cast(f16_t, (uint16_t)(w >> 16));
+  else return __builtin_bit_cast(float, w & 0xffff0000u);
+}
+template <bool HALF>
+__device__ __forceinline__ float dot2_f32(uint32_t a, uint32_t b, float c) {
+  if constexpr (HALF) return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, a), __builtin_bit_cast(f16x2_t, b), c, false);
+  else return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
+}
+template <bool HALF>
+__device__ __forceinline__ uint16_t round_out(float v) {
+  if constexpr (HALF) return __builtin_bit_cast(uint16_t, (f16_t)v);
+  else return f32_to_bf16(v);
+}
+template <bool HALF>
+__device__ __forceinline__ uint32_t round_out_x2(float lo, float hi) {
+  if constexpr (HALF) return pack_f16x2(lo, hi);
+  else return pack_bf16x2(lo, hi);
+}
+
 // W is the (work-group uniform) start of the expert's column block; coff the thread's column offset in elements.
 // One step = one 16-byte load per thread = KR weight rows per work-group.
 template <int KR>
@@ -35,21 +66,26 @@ __device__ __forceinline__ u32x4_t load_step(const bf16_bits* W, uint32_t coff, 
   return __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(W + off));
 }
 
-template <int KR, int R>
+template <int KR, int R, bool HALF>
 __device__ __forceinline__ void fma_step(float (&acc)[kRows][8], const u32x4_t w, const u32x2_t* xs, int step, int kr,
                                          int k) {
   const int kk_raw = step * KR + kr;
   const uint32_t live = kk_raw < k ? 0xffffffffu : 0u;  // rows past k contribute nothing
   const u32x2_t xp = xs[imin(kk_raw, k - 1)];          // the kRows activations for contraction index kk, as bf16
   float xv[kRows];
-  xv[0] = __builtin_bit_cast(float, (xp[0] << 16) & live);
-  xv[1] = __builtin_bit_cast(float, xp[0] & 0xffff0000u & live);
-  xv[2] = __builtin_bit_cast(float, (xp[1] << 16) & live);
-  xv[3] = __builtin_bit_cast(float, xp[1] & 0xffff0000u & live);
+  if constexpr (HALF) {
+    const uint32_t x0 = xp[0] & live, x1 = xp[1] & live;
+    xv[0] = lo_f32<true>(x0); xv[1] = hi_f32<true>(x0); xv[2] = lo_f32<true>(x1); xv[3] = hi_f32<true>(x1);
+  } else {
+    xv[0] = __builtin_bit_cast(float, (xp[0] << 16) & live);
+    xv[1] = __builtin_bit_cast(float, xp[0] & 0xffff0000u & live);
+    xv[2] = __builtin_bit_cast(float, (xp[1] << 16) & live);
+    xv[3] = __builtin_bit_cast(float, xp[1] & 0xffff0000u & live);
+  }
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    const float lo = __builtin_bit_cast(float, w[e] << 16);
-    const float hi = __builtin_bit_cast(float, w[e] & 0xffff0000u);
+    const float lo = lo_f32<HALF>(w[e]);
+    const float hi = hi_f32<HALF>(w[e]);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       acc[r][2 * e] = __builtin_fmaf(xv[r], lo, acc[r][2 * e]);
@@ -60,20 +96,20 @@ __device__ __forceinline__ void fma_step(float (&acc)[kRows][8], const u32x4_t w
 
 // The streaming loop for R live rows: a ring of kDepth loads per thread, each refilled with the load kDepth steps
 // ahead as soon as it is consumed.
-template <int KR, int R>
+template <int KR, int R, bool HALF>
 __device__ __forceinline__ void stream_weights(float (&acc)[kRows][8], u32x4_t (&w)[kDepth], const bf16_bits* W,
                                                uint32_t coff, const u32x2_t* xs, int kr, int k, int n) {
   const int nsteps = (k + KR - 1) / KR;
   for (int base = 0; base < nsteps; base += kDepth) {
 #pragma unroll
     for (int u = 0; u < kDepth; ++u) {
-      fma_step<KR, R>(acc, w[u], xs, base + u, kr, k);
+      fma_step<KR, R, HALF>(acc, w[u], xs, base + u, kr, k);
       w[u] = load_step<KR>(W, coff, base + kDepth + u, kr, k, n);
     }
   }
 }
 
-template <int NB>
+template <int NB, bool HALF>
 __global__ __launch_bounds__(kThreads, 3) void gmm_decode_kernel(DecodeArgs p) {
   static_assert(kRows == 4, "activations are staged as one 8-byte word per contraction index");
   constexpr int TPR = NB / 8;          // threads across one weight row segment
@@ -166,10 +202,10 @@ __global__ __launch_bounds__(kThreads, 3) void gmm_decode_kernel(DecodeArgs p) {
     }
     // a group rarely has more than one or two rows here: only the live ones cost vector-ALU work
     switch (nr) {
-      case 1: stream_weights<KR, 1>(acc, w, W, coff, xs, kr, p.k, p.n); break;
-      case 2: stream_weights<KR, 2>(acc, w, W, coff, xs, kr, p.k, p.n); break;
-      case 3: stream_weights<KR, 3>(acc, w, W, coff, xs, kr, p.k, p.n); break;
-      default: stream_weights<KR, 4>(acc, w, W, coff, xs, kr, p.k, p.n); break;
+      case 1: stream_weights<KR, 1, HALF>(acc, w, W, coff, xs, kr, p.k, p.n); break;
+      case 2: stream_weights<KR, 2, HALF>(acc, w, W, coff, xs, kr, p.k, p.n); break;
+      case 3: stream_weights<KR, 3, HALF>(acc, w, W, coff, xs, kr, p.k, p.n); break;
+      default: stream_weights<KR, 4, HALF>(acc, w, W, coff, xs, kr, p.k, p.n); break;
     }
 
     // reduce over the weight rows: first the row-slots inside a wave, then the 4 waves through LDS
@@ -195,17 +231,17 @@ __global__ __launch_bounds__(kThreads, 3) void gmm_decode_kernel(DecodeArgs p) {
         float v = 0.f;
 #pragma unroll
         for (int w2 = 0; w2 < kThreads / 64; ++w2) v += part[(w2 * kRows + r) * NB + c];
-        p.y[(size_t)(row0 + rc + r) * p.n + col0 + c] = f32_to_bf16(v);
+        p.y[(size_t)(row0 + rc + r) * p.n + col0 + c] = round_out<HALF>(v);
       }
     }
   }
 }
 
-template <int NB>
+template <int NB, bool HALF>
 int launch_nb(hipStream_t s, const DecodeArgs& a) {
   const int n_blocks = (a.n + NB - 1) / NB;
   const size_t lds = (size_t)a.k * 8 + (size_t)(kThreads / 64) * kRows * NB * sizeof(float);
-  auto kern = gmm_decode_kernel<NB>;
+  auto kern = gmm_decode_kernel<NB, HALF>;
   if (lds > 64 * 1024) {
     const int rc = (int)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -245,21 +281,26 @@ __device__ __forceinline__ u32x4_t load_row_step(const bf16_bits* W, uint32_t co
   return __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(W + (uint32_t)kk * (uint32_t)n + coff));
 }
 
-template <int R>
+template <int R, bool HALF>
 __device__ __forceinline__ void fma_row_step(float (&acc)[kRows][8], const u32x4_t w, const u32x2_t* xs, int step, int rps,
                                              int kr, int klen) {
   const int kk_raw = step * rps + kr;
   const uint32_t live = kk_raw < klen ? 0xffffffffu : 0u;
   const u32x2_t xp = xs[imin(kk_raw, klen - 1)];
   float xv[kRows];
-  xv[0] = __builtin_bit_cast(float, (xp[0] << 16) & live);
-  xv[1] = __builtin_bit_cast(float, xp[0] & 0xffff0000u & live);
-  xv[2] = __builtin_bit_cast(float, (xp[1] << 16) & live);
-  xv[3] = __builtin_bit_cast(float, xp[1] & 0xffff0000u & live);
+  if constexpr (HALF) {
+    const uint32_t x0 = xp[0] & live, x1 = xp[1] & live;
+    xv[0] = lo_f32<true>(x0); xv[1] = hi_f32<true>(x0); xv[2] = lo_f32<true>(x1); xv[3] = hi_f32<true>(x1);
+  } else {
+    xv[0] = __builtin_bit_cast(float, (xp[0] << 16) & live);
+    xv[1] = __builtin_bit_cast(float, xp[0] & 0xffff0000u & live);
+    xv[2] = __builtin_bit_cast(float, (xp[1] << 16) & live);
+    xv[3] = __builtin_bit_cast(float, xp[1] & 0xffff0000u & live);
+  }
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    const float lo = __builtin_bit_cast(float, w[e] << 16);
-    const float hi = __builtin_bit_cast(float, w[e] & 0xffff0000u);
+    const float lo = lo_f32<HALF>(w[e]);
+    const float hi = hi_f32<HALF>(w[e]);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       acc[r][2 * e] = __builtin_fmaf(xv[r], lo, acc[r][2 * e]);
@@ -268,14 +309,14 @@ __device__ __forceinline__ void fma_row_step(float (&acc)[kRows][8], const u32x4
   }
 }
 
-template <int R>
+template <int R, bool HALF>
 __device__ __forceinline__ void stream_rows(float (&acc)[kRows][8], u32x4_t (&w)[kRowsDepth], const bf16_bits* W, uint32_t coff,
                                             const u32x2_t* xs, int rps, int kr, int klen, int n) {
   const int nsteps = (klen + rps - 1) / rps;
   for (int base = 0; base < nsteps; base += kRowsDepth) {
 #pragma unroll
     for (int u = 0; u < kRowsDepth; ++u) {
-      fma_row_step<R>(acc, w[u], xs, base + u, rps, kr, klen);
+      fma_row_step<R, HALF>(acc, w[u], xs, base + u, rps, kr, klen);
       w[u] = load_row_step(W, coff, base + kRowsDepth + u, rps, kr, klen, n);
     }
   }
@@ -293,8 +334,6 @@ constexpr int kWideSeg = 1024;   // contraction indices staged at a time: (kWide
 constexpr int kWideStage = 4;    // activation words a thread stages per round trip
 constexpr int kXsBytes = ((kWideSeg >> 1) + 1) * kWideRows * 4;
 
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-
 // Weight rows 2 * (step * rps + kr) and the one after it, clamped to the segment (rows past klen, which is even,
 // re-read its last two rows; their activations are read from the all-zero entry).
 __device__ __forceinline__ void load_row_pair(u32x4_t& even, u32x4_t& odd, const bf16_bits* W, uint32_t coff, int step, int rps,
@@ -305,7 +344,7 @@ __device__ __forceinline__ void load_row_pair(u32x4_t& even, u32x4_t& odd, const
   odd = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(W + off + (uint32_t)n));
 }
 
-template <int R>
+template <int R, bool HALF>
 __device__ __forceinline__ void fma_row_pair(float (&acc)[kWideRows][8], const u32x4_t even, const u32x4_t odd,
                                              const u32x4_t* xs, int step, int rps, int kr, int pairs) {
   const int pj = step * rps + kr;
@@ -323,14 +362,13 @@ __device__ __forceinline__ void fma_row_pair(float (&acc)[kWideRows][8], const u
     const uint32_t hi = __builtin_amdgcn_perm(odd[e], even[e], 0x07060302u);  // (W[kk][2e + 1], W[kk + 1][2e + 1])
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const bf16x2_t xr = __builtin_bit_cast(bf16x2_t, xv[r]);
-      acc[r][2 * e] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, lo), xr, acc[r][2 * e], false);
-      acc[r][2 * e + 1] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, hi), xr, acc[r][2 * e + 1], false);
+      acc[r][2 * e] = dot2_f32<HALF>(lo, xv[r], acc[r][2 * e]);
+      acc[r][2 * e + 1] = dot2_f32<HALF>(hi, xv[r], acc[r][2 * e + 1]);
     }
   }
 }
 
-template <int R>
+template <int R, bool HALF>
 __device__ __forceinline__ void stream_row_pairs(float (&acc)[kWideRows][8], u32x4_t (&w)[2 * kPairDepth], const bf16_bits* W,
                                                  uint32_t coff, const u32x4_t* xs, int rps, int kr, int klen, int n) {
   const int nsteps = (klen + 2 * rps - 1) / (2 * rps);
@@ -338,7 +376,7 @@ __device__ __forceinline__ void stream_row_pairs(float (&acc)[kWideRows][8], u32
   for (int base = 0; base < nsteps; base += kPairDepth) {
 #pragma unroll
     for (int u = 0; u < kPairDepth; ++u) {
-      fma_row_pair<R>(acc, w[2 * u], w[2 * u + 1], xs, base + u, rps, kr, pairs);
+      fma_row_pair<R, HALF>(acc, w[2 * u], w[2 * u + 1], xs, base + u, rps, kr, pairs);
       // Keep every refill where it is written: sunk to the end of the iteration, the loads would all wait for the last
       // pair and the ring would run empty once per iteration.
       __builtin_amdgcn_sched_barrier(0);
@@ -349,6 +387,7 @@ __device__ __forceinline__ void stream_row_pairs(float (&acc)[kWideRows][8], u32
 }
 
 // One pass of nr = 1 .. 8 rows (rows row_first ..) of a piece: its sums into part[kr][r][n] of the loader threads.
+template <bool HALF>
 __device__ __forceinline__ void wide_pass(const DecodeArgs& p, int rps, int unit, int gi, int row_first, int nr, int k0,
                                           int klen_all, int tid, int tc, int kr, bool loader, unsigned char* smem_raw,
                                           float* part) {
@@ -391,14 +430,14 @@ __device__ __forceinline__ void wide_pass(const DecodeArgs& p, int rps, int unit
     __syncthreads();
     if (loader) {
       switch (nr) {
-        case 1: stream_row_pairs<1>(acc, w, W, coff, xs, rps, kr, klen, p.n); break;
-        case 2: stream_row_pairs<2>(acc, w, W, coff, xs, rps, kr, klen, p.n); break;
-        case 3: stream_row_pairs<3>(acc, w, W, coff, xs, rps, kr, klen, p.n); break;
-        case 4: stream_row_pairs<4>(acc, w, W, coff, xs, rps, kr, klen, p.n); break;
-        case 5: stream_row_pairs<5>(acc, w, W, coff, xs, rps, kr, klen, p.n); break;
-        case 6: stream_row_pairs<6>(acc, w, W, coff, xs, rps, kr, klen, p.n); break;
-        case 7: stream_row_pairs<7>(acc, w, W, coff, xs, rps, kr, klen, p.n); break;
-        default: stream_row_pairs<8>(acc, w, W, coff, xs, rps, kr, klen, p.n); break;
+        case 1: stream_row_pairs<1, HALF>(acc, w, W, coff, xs, rps, kr, klen, p.n); break;
+        case 2: stream_row_pairs<2, HALF>(acc, w, W, coff, xs, rps, kr, klen, p.n); break;
+        case 3: stream_row_pairs<3, HALF>(acc, w, W, coff, xs, rps, kr, klen, p.n); break;
+        case 4: stream_row_pairs<4, HALF>(acc, w, W, coff, xs, rps, kr, klen, p.n); break;
+        case 5: stream_row_pairs<5, HALF>(acc, w, W, coff, xs, rps, kr, klen, p.n); break;
+        case 6: stream_row_pairs<6, HALF>(acc, w, W, coff, xs, rps, kr, klen, p.n); break;
+        case 7: stream_row_pairs<7, HALF>(acc, w, W, coff, xs, rps, kr, klen, p.n); break;
+        default: stream_row_pairs<8, HALF>(acc, w, W, coff, xs, rps, kr, klen, p.n); break;
       }
     }
   }
@@ -416,7 +455,7 @@ __device__ __forceinline__ void wide_pass(const DecodeArgs& p, int rps, int unit
 }
 
 
-template <bool WIDE>
+template <bool WIDE, bool HALF>
 __global__ __launch_bounds__(kThreads, 2) void gmm_rows_kernel(DecodeArgs p, RowsGeom q, RowsHeader* __restrict__ header,
                                                                float* __restrict__ partials) {
   __shared__ int32_t wave_cnt[3][kThreads / 64];
@@ -521,7 +560,7 @@ __global__ __launch_bounds__(kThreads, 2) void gmm_rows_kernel(DecodeArgs p, Row
     if constexpr (WIDE) {
       for (int rc = 0; rc < rows; rc += kWideRows) {
         const int nr = imin(kWideRows, rows - rc);
-        wide_pass(p, q.rps, unit, gi, row0 + rc, nr, k0, klen_all, tid, tc, kr, loader, smem_raw, part);
+        wide_pass<HALF>(p, q.rps, unit, gi, row0 + rc, nr, k0, klen_all, tid, tc, kr, loader, smem_raw, part);
         __syncthreads();
         for (int idx = tid; idx < nr * p.n; idx += kThreads) {
           const int r = idx / p.n, col = idx - r * p.n;
@@ -560,10 +599,10 @@ __global__ __launch_bounds__(kThreads, 2) void gmm_rows_kernel(DecodeArgs p, Row
         __syncthreads();
         if (loader) {
           switch (nr) {
-            case 1: stream_rows<1>(acc, w, W, coff, xs, q.rps, kr, klen, p.n); break;
-            case 2: stream_rows<2>(acc, w, W, coff, xs, q.rps, kr, klen, p.n); break;
-            case 3: stream_rows<3>(acc, w, W, coff, xs, q.rps, kr, klen, p.n); break;
-            default: stream_rows<4>(acc, w, W, coff, xs, q.rps, kr, klen, p.n); break;
+            case 1: stream_rows<1, HALF>(acc, w, W, coff, xs, q.rps, kr, klen, p.n); break;
+            case 2: stream_rows<2, HALF>(acc, w, W, coff, xs, q.rps, kr, klen, p.n); break;
+            case 3: stream_rows<3, HALF>(acc, w, W, coff, xs, q.rps, kr, klen, p.n); break;
+            default: stream_rows<4, HALF>(acc, w, W, coff, xs, q.rps, kr, klen, p.n); break;
           }
         }
       }
@@ -633,8 +672,9 @@ __device__ __forceinline__ float wave_sums(float (&v)[V], int lane) {
 // activations are widened to bf16 as they are staged (two 16-byte entries per chunk, the chunk's lower and upper eight),
 // the weights as they are used (one v_cvt_scalef32_pk_bf16_fp8 per pair, once per block of weight rows and shared
 // by the token rows), and the same v_dot2_f32_bf16 multiplies them - exactly, every e4m3 value being a bf16 value.
-template <int RMAX, bool F8>
+template <int RMAX, bool F8, bool HALF>
 __global__ __launch_bounds__(kThreads, 2) void gmm_rows_t_kernel(DecodeArgs p, int wgs) {
+  static_assert(!(F8 && HALF), "float8 operands are widened to bf16");
   constexpr int EB = F8 ? 1 : 2;     // bytes per element of x and A
   constexpr int EPC = 16 / EB;       // elements per 16-byte chunk
   constexpr int XE = F8 ? 2 : 1;     // staged 16-byte entries per chunk and token row
@@ -833,10 +873,10 @@ __global__ __launch_bounds__(kThreads, 2) void gmm_rows_t_kernel(DecodeArgs p, i
 #pragma unroll
                 for (int b = 0; b < kTBlock; ++b) {
                   float a = acc[b][r];
-                  a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, wp[b][4 * h + 0]), __builtin_bit_cast(bf16x2_t, x0), a, false);
-                  a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, wp[b][4 * h + 1]), __builtin_bit_cast(bf16x2_t, x1), a, false);
-                  a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, wp[b][4 * h + 2]), __builtin_bit_cast(bf16x2_t, x2), a, false);
-                  a = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, wp[b][4 * h + 3]), __builtin_bit_cast(bf16x2_t, x3), a, false);
+                  a = dot2_f32<HALF>(wp[b][4 * h + 0], x0, a);
+                  a = dot2_f32<HALF>(wp[b][4 * h + 1], x1, a);
+                  a = dot2_f32<HALF>(wp[b][4 * h + 2], x2, a);
+                  a = dot2_f32<HALF>(wp[b][4 * h + 3], x3, a);
                   acc[b][r] = a;
                 }
               }
@@ -854,7 +894,7 @@ __global__ __launch_bounds__(kThreads, 2) void gmm_rows_t_kernel(DecodeArgs p, i
               const int idx = lane / RUN;
               const int b = idx / RMAX, r = idx - b * RMAX;
               if (lane % RUN == 0 && r < nr)
-                p.y[(size_t)(row0 + rc + r) * p.n + (j_begin + kTBlock * (wave + 4 * i) + b)] = f32_to_bf16(mine);
+                p.y[(size_t)(row0 + rc + r) * p.n + (j_begin + kTBlock * (wave + 4 * i) + b)] = round_out<HALF>(mine);
               q = 0; ++i;
             }
           }
@@ -869,6 +909,7 @@ __global__ __launch_bounds__(kThreads, 2) void gmm_rows_t_kernel(DecodeArgs p, i
 
 // y[row, :] = sum over the pieces of partials[row, piece, :] for rows below sum(group_sizes), zero above.
 // Work-group = (row, block of 256 columns); thread = (8 columns, one of 8 piece lanes).
+template <bool HALF>
 __global__ __launch_bounds__(kThreads) void gmm_rows_finish_kernel(DecodeArgs p, const RowsHeader* __restrict__ header,
                                                                    const float* __restrict__ partials) {
   __shared__ float sums[8][32][8];
@@ -900,7 +941,7 @@ __global__ __launch_bounds__(kThreads) void gmm_rows_finish_kernel(DecodeArgs p,
     }
     u32x4_t out;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) out[e] = pack_bf16x2(t[2 * e], t[2 * e + 1]);
+    for (int e = 0; e < 4; ++e) out[e] = round_out_x2<HALF>(t[2 * e], t[2 * e + 1]);
     *reinterpret_cast<u32x4_t*>(p.y + (size_t)row * p.n + col) = out;
   }
 }
@@ -910,9 +951,9 @@ __global__ __launch_bounds__(kThreads) void gmm_rows_finish_kernel(DecodeArgs p,
 int launch_gmm_decode(hipStream_t s, const DecodeArgs& a, int nb) {
   if (a.m <= 0 || a.n <= 0 || a.g <= 0) return hipSuccess;
   switch (nb) {
-    case 32: return launch_nb<32>(s, a);
-    case 64: return launch_nb<64>(s, a);
-    case 128: return launch_nb<128>(s, a);
+    case 32: return a.half ? launch_nb<32, true>(s, a) : launch_nb<32, false>(s, a);
+    case 64: return a.half ? launch_nb<64, true>(s, a) : launch_nb<64, false>(s, a);
+    case 128: return a.half ? launch_nb<128, true>(s, a) : launch_nb<128, false>(s, a);
     default: return hipErrorInvalidValue;
   }
 }
@@ -924,17 +965,17 @@ size_t gmm_rows_workspace_bytes(int m, int n, int pieces) {
 
 namespace {
 
-template <bool WIDE>
+template <bool WIDE, bool HALF>
 int launch_rows(hipStream_t s, const DecodeArgs& a, RowsGeom q, RowsHeader* header, float* partials) {
   q.min_rows = WIDE ? q.rps * 2 * kPairDepth * 2 : q.rps * kRowsDepth * 2;
   const size_t lds = WIDE ? (size_t)kXsBytes + (size_t)q.rps * kWideRows * a.n * sizeof(float)
                           : (size_t)kMaxSeg * 8 + (size_t)q.rps * kRows * a.n * sizeof(float);
   if (lds > 64 * 1024) {
-    const int rc = (int)hipFuncSetAttribute(reinterpret_cast<const void*>(gmm_rows_kernel<WIDE>),
+    const int rc = (int)hipFuncSetAttribute(reinterpret_cast<const void*>(gmm_rows_kernel<WIDE, HALF>),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (rc != hipSuccess) return rc;
   }
-  hipLaunchKernelGGL(gmm_rows_kernel<WIDE>, dim3(q.wgs), dim3(kThreads), lds, s, a, q, header, partials);
+  hipLaunchKernelGGL((gmm_rows_kernel<WIDE, HALF>), dim3(q.wgs), dim3(kThreads), lds, s, a, q, header, partials);
   return (int)hipGetLastError();
 }
 
@@ -955,10 +996,12 @@ int launch_gmm_rows(hipStream_t s, const DecodeArgs& a, int num_cus, void* works
   float* partials = reinterpret_cast<float*>(static_cast<char*>(workspace) + 256);
   // More than one row per group on average: some group has more than the four rows a narrow pass takes, and the
   // wide passes stream its weights once where the narrow ones would twice.
-  const int rc = a.m > a.g ? launch_rows<true>(s, a, q, header, partials) : launch_rows<false>(s, a, q, header, partials);
+  const int rc = a.m > a.g ? (a.half ? launch_rows<true, true>(s, a, q, header, partials) : launch_rows<true, false>(s, a, q, header, partials))
+                           : (a.half ? launch_rows<false, true>(s, a, q, header, partials) : launch_rows<false, false>(s, a, q, header, partials));
   if (rc != hipSuccess) return rc;
   const int col_blocks = (a.n + 255) / 256;
-  hipLaunchKernelGGL(gmm_rows_finish_kernel, dim3(a.m * col_blocks), dim3(kThreads), 0, s, a, header, partials);
+  if (a.half) hipLaunchKernelGGL(gmm_rows_finish_kernel<true>, dim3(a.m * col_blocks), dim3(kThreads), 0, s, a, header, partials);
+  else hipLaunchKernelGGL(gmm_rows_finish_kernel<false>, dim3(a.m * col_blocks), dim3(kThreads), 0, s, a, header, partials);
   return (int)hipGetLastError();
 }
 
@@ -982,11 +1025,15 @@ int launch_gmm_rows_t(hipStream_t s, const DecodeArgs& a, int num_cus, bool f8) 
   const size_t lds = (size_t)(wide ? 8 : 4) * kpad * 2;
   if (lds > (size_t)kTMaxLds) return hipErrorInvalidValue;
   if (f8) {
-    if (wide) hipLaunchKernelGGL((gmm_rows_t_kernel<8, true>), dim3(wgs), dim3(kThreads), lds, s, a, wgs);
-    else hipLaunchKernelGGL((gmm_rows_t_kernel<4, true>), dim3(wgs), dim3(kThreads), lds, s, a, wgs);
+    if (a.half) return hipErrorInvalidValue;
+    if (wide) hipLaunchKernelGGL((gmm_rows_t_kernel<8, true, false>), dim3(wgs), dim3(kThreads), lds, s, a, wgs);
+    else hipLaunchKernelGGL((gmm_rows_t_kernel<4, true, false>), dim3(wgs), dim3(kThreads), lds, s, a, wgs);
+  } else if (a.half) {
+    if (wide) hipLaunchKernelGGL((gmm_rows_t_kernel<8, false, true>), dim3(wgs), dim3(kThreads), lds, s, a, wgs);
+    else hipLaunchKernelGGL((gmm_rows_t_kernel<4, false, true>), dim3(wgs), dim3(kThreads), lds, s, a, wgs);
   } else {
-    if (wide) hipLaunchKernelGGL((gmm_rows_t_kernel<8, false>), dim3(wgs), dim3(kThreads), lds, s, a, wgs);
-    else hipLaunchKernelGGL((gmm_rows_t_kernel<4, false>), dim3(wgs), dim3(kThreads), lds, s, a, wgs);
+    if (wide) hipLaunchKernelGGL((gmm_rows_t_kernel<8, false, false>), dim3(wgs), dim3(kThreads), lds, s, a, wgs);
+    else hipLaunchKernelGGL((gmm_rows_t_kernel<4, false, false>), dim3(wgs), dim3(kThreads), lds, s, a, wgs);
   }
   return (int)hipGetLastError();
 }

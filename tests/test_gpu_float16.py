@@ -192,4 +192,40 @@ def test_float16_default_is_the_four_wave_core_on_large_shapes():
         assert vs[_capi.default_plan(op, *shape, _capi.RD_DTYPE_F16).variant] == "hw256x256x32_w2x2_s5"
     small = _capi.default_plan(_capi.OP_GMM, 300, 128, 256, 4, _capi.RD_DTYPE_F16)
     assert vs[small.variant].startswith("h") and small.decode_nb == 0
-    assert _capi.default_plan(_capi.OP_GMM, 64, 2048, 768, 128, _capi.RD_DTYPE_F16).decode_nb == 0   # no streaming kernels
+    assert _capi.default_plan(_capi.OP_GMM, 64, 2048, 768, 128, _capi.RD_DTYPE_F16).decode_nb == _capi.RD_DECODE_ROWS
+    assert _capi.default_plan(_capi.OP_GMM_TRANS, 64, 2048, 768, 128, _capi.RD_DTYPE_F16).decode_nb == _capi.RD_DECODE_ROWS
+
+
+@pytest.mark.parametrize("m,hot", [(48, None), (200, None), (256, 5)], ids=["m48", "m200", "m256_one_group"])
+def test_float16_streaming_kernels(m, hot):
+    """A few rows per group: the streaming kernels in float16 - whole-row slices with 4 and with 8 rows per pass and
+    their finishing kernel, the form for weights stored [g, n, k], the column-strip kernel at its three widths - under
+    the default plan and forced, with empty groups, a zero tail, and all rows piled into one group."""
+    from gpu_ragged_dot_amd import ops
+    print("f16 streaming", m, hot, flush=True)
+    k, n, g = 1024, 512, 64
+    rng = np.random.default_rng(m)
+    if hot is None:
+        gs = oracle.generate_group_sizes(m, g, m - 5)
+        gs[rng.random(g) < 0.3] = 0
+    else:
+        gs = np.zeros(g, np.int32)
+        gs[hot] = m - 5
+    live = int(gs.sum())
+    lhs = oracle.round_to(rng.normal(size=(m, k)).astype(np.float32), "float16")
+    rhs = oracle.round_to((rng.normal(size=(g, k, n)) / np.sqrt(k)).astype(np.float32), "float16")
+    ref = oracle.gmm(lhs, rhs, gs, out_dtype="float16")
+    hp = dict(block_m=64, block_k=64, block_n=64, interpret=False, compute_dtype=None, acc_dtype=torch.float32, chunk_m=512)
+    x_t, A_t, gs_t = _dev(lhs), _dev(rhs), torch.from_numpy(gs)
+    At_t = A_t.mT.contiguous()
+    assert _capi.default_plan(_capi.OP_GMM, m, k, n, g, _capi.RD_DTYPE_F16).decode_nb == _capi.RD_DECODE_ROWS
+    plans = [None, _capi.Plan(-1, 0, _capi.RD_DECODE_ROWS), _capi.Plan(-1, 0, 32), _capi.Plan(-1, 0, 64), _capi.Plan(-1, 0, 128)]
+    for plan in plans:
+        o = ops._gmm_fwd(x_t, A_t, gs_t, **hp, trans_rhs=False, plan=plan)
+        assert o.dtype == torch.float16
+        util.assert_close_rows(util.to_np(o), ref, live, F16_EPS, f"plan {plan}")
+        assert not np.any(util.to_np(o)[live:])
+    for plan in (None, _capi.Plan(-1, 0, _capi.RD_DECODE_ROWS)):
+        o = ops._gmm_fwd(x_t, At_t, gs_t, **hp, trans_rhs=True, plan=plan)
+        util.assert_close_rows(util.to_np(o), ref, live, F16_EPS, f"weights transposed, plan {plan}")
+        assert not np.any(util.to_np(o)[live:])
