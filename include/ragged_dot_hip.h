@@ -46,8 +46,9 @@ extern "C" {
  * float8 has the one for weights stored [g, n, k] (trans_rhs, decode_nb = RD_DECODE_ROWS, k % 16 == 0; rd_default_plan
  * picks it up to one row per group on average); the K-split of rd_plan.split_k on the first path only.
  * RD_DTYPE_F16: float16 (IEEE half) arrays - the reference takes whatever element type its arrays have - multiplied on
- * the float16 matrix-core instruction with fp32 accumulation, float16 out (nearest even).  Tile kernels of the
- * register-staged kind for any shape; no streaming kernels, no K-split. */
+ * the float16 matrix-core instruction with fp32 accumulation, float16 out (nearest even).  Everything bfloat16 has
+ * except the smaller direct-to-LDS tile shapes: the four-wave 256 x 256 core with the K-split, register-staged tiles for
+ * any shape, the streaming kernels for a few rows per group, the routing kernels. */
 enum rd_dtype { RD_DTYPE_BF16 = 0, RD_DTYPE_F32 = 1, RD_DTYPE_F32_BF16 = 2, RD_DTYPE_F8E4M3_BF16 = 3, RD_DTYPE_F16 = 4 };
 
 #define RD_DECODE_ROWS (-1) /* rd_plan.decode_nb: the streaming kernel that cuts each expert's weights into whole-row slices */
