@@ -233,7 +233,8 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
     sk.part = part;
   }
   const int band = uniform(p.tile2band[t / p.n_tiles]);
-  const int band_row0 = band >> kBandShift, band_rows = band & kBandMaxRows;
+  const bool deferred = (band & kBandDeferred) != 0;  // a short last row tile the map has moved behind all other tiles
+  const int band_row0 = (band & ~kBandDeferred) >> kBandShift, band_rows = band & kBandMaxRows;
   const int w = t - band_row0 * p.n_tiles;
   const int nj = w / band_rows;
   const int mi = band_row0 + (w - nj * band_rows);
@@ -258,10 +259,11 @@ __global__ __launch_bounds__(C::NT, C::WAVES_PER_EU) void gmm_kernel(GmmArgs p) 
     const E* Bp = TRANS_RHS ? pA + (size_t)gl * p.n * p.k + (size_t)col0 * p.k + k0
                             : pA + (size_t)gl * p.k * p.n + (size_t)k0 * p.n + col0;
     if constexpr (IsW4<C>::value && C::A_KMAJOR) {
-      // Only for a group's single row tile.  The short last tile of a longer group stays on the tall routine: run
+      // For a group's single row tile, and for the short last tile of a longer group where the scheduling map has moved
+      // it behind all other tiles (into the K-split last round).  Left in its group's run such a tile must stay on the tall routine: run
       // through the short one it finishes early, the tiles dealt next start out of step with the rest of their block,
       // and the block's operand slabs are fetched into L2 twice (measured: +1 GB of fetches per launch, no time gained).
-      if (rows <= kMidRows && it == 0) {
+      if (rows <= kMidRows && (it == 0 || deferred)) {
         typedef typename ShortTileCfg<C, kShortRows>::type S;
         typedef typename ShortTileCfg<C, kMidRows>::type M;
         static_assert(S::LDS_BYTES <= C::LDS_BYTES && S::NT == C::NT && S::BN == C::BN, "the short routine runs in the tall one's launch");

@@ -9,6 +9,7 @@ namespace rd {
 // tile2band entries: (first row tile of the band << kBandShift) | rows of the band.
 constexpr int kBandShift = 7;
 constexpr int kBandMaxRows = (1 << kBandShift) - 1;
+constexpr int kBandDeferred = 1 << 30;  // mark of a short last row tile listed behind all other tiles (see launch_sched_map)
 
 // Arrays as in the reference's GMMGroupLookupMetadata (gpu_ragged_dot.py:60-90); tile2group / tile2it hold
 // ceil(m / chunk) + g entries.  `counters` (may be null) are n_counters int32 cleared by the same launch.
@@ -27,11 +28,16 @@ constexpr int kBandMaxRows = (1 << kBandShift) - 1;
 // 1.90; an exact sort by rows gives the same, classes of 64 or 128 rows half of it or nothing, long groups merely moved
 // to the front nothing).  Where two groups' tiles share an XCD the order the groups come in mixes long and short
 // tiles and is the better one (128 groups with Zipf lengths, k 2048, n 4096: 0.84 -> 0.88 ms), hence an option of the plan.
+// `defer_rows` > 0 (internal maps of gmm launches only, needs tile2band): the last row tile of a group of two or more
+// row tiles, when it holds at most defer_rows rows, is listed behind all other tiles instead of behind its group's - as a
+// band of its own, marked kBandDeferred - provided all such tiles then lie in the launch's partly filled last round
+// (defer_cus tiles run at a time) and that round holds at most defer_slots / 2 tiles, i.e. is cut along K.
 int launch_sched_map(hipStream_t s, const int32_t* group_sizes, int g, int m, int chunk, int32_t* group_offsets,
                      int32_t* tile2group, int32_t* tile2it, int32_t* total_tiles, int32_t* counters = nullptr,
                      int n_counters = 0, int32_t* tile2band = nullptr, int band_rows = 1, int32_t* block_order = nullptr,
                      int n_blocks = 0, int per_block = 1, int n_tiles = 1, int long_rows = 0,
-                     int32_t* group_order = nullptr, int order_first = 0, int order_count = 0);
+                     int32_t* group_order = nullptr, int order_first = 0, int order_count = 0, int defer_rows = 0,
+                     int defer_cus = 0, int defer_slots = 0);
 
 // Which block the i-th block position of a gmm launch takes from the two lists of block_order.  Positions are dealt to
 // the 8 XCDs round-robin (position i runs on XCD i mod 8), so the launch is a sequence of rounds of 8.  The long groups'

@@ -54,22 +54,63 @@ __global__ __launch_bounds__(kSchedThreads) void sched_map_kernel(const int32_t*
                                                                   int32_t* __restrict__ block_order, int n_blocks,
                                                                   int per_block, int n_tiles, int long_rows,
                                                                   int32_t* __restrict__ group_order, int order_first,
-                                                                  int order_count) {
+                                                                  int order_count, int defer_rows, int defer_cus,
+                                                                  int defer_slots) {
   // arrival counters of the K-split tiles of the launch that follows start at zero
   for (int i = threadIdx.x; i < n_counters; i += kSchedThreads) counters[i] = 0;
   __shared__ uint32_t wave_a[kSchedWaves], wave_b[kSchedWaves];
   __shared__ int32_t incl[kSchedThreads];  // inclusive tile-count scan of the current slab of groups
+  __shared__ int32_t incl_d[kSchedThreads], tiles_of[kSchedThreads];  // deferred tiles: their scan, and every group's tile count
   const int tid = threadIdx.x;
-  uint32_t carry_rows = 0, carry_tiles = 0;
+  uint32_t carry_rows = 0, carry_tiles = 0, carry_def = 0;
+
+  // defer_rows > 0 (gmm launches of the cores that have the streaming routines, when the last round of tiles is cut along
+  // K; never the map rd_sched_map returns): the last row tile of a group of several row tiles, when it holds at most
+  // defer_rows rows, may be taken out of its group's run of tiles and listed behind all other tiles, as a band of its
+  // own with the kBandDeferred mark.  That is done when all such tiles then fall into the partly filled last round of
+  // the launch (defer_cus tiles run at a time) and that round is cut along K (at most defer_slots / 2 tiles in it): the
+  // rounds before it then hold whole tiles of full height only - the layout of a dense product - and the pieces of the
+  // last round, which run alone at the end of the launch either way, go through the streaming routines instead of the
+  // tall one.  Anywhere else a tile moved out of its group's run would cost a pass of its own over the group's weights.
+  bool defer_on = false;
+  auto deferred = [&](int32_t sz, int32_t bpg) {
+    return defer_on && bpg >= 2 && sz - (bpg - 1) * chunk <= defer_rows ? 1 : 0;
+  };
+  uint32_t total_regular = 0;
+  if (defer_rows > 0 && defer_cus > 0) {  // count the candidates and all tiles, then decide
+    uint32_t all = 0, cand = 0;
+    defer_on = true;
+    for (int base = 0; base < g; base += kSchedThreads) {
+      const int gi = base + tid;
+      const int32_t sz = gi < g ? gs[gi] : 0;
+      const int32_t bpg = gi < g ? floor_div(sz + chunk - 1, chunk) : 0;
+      uint32_t a = (uint32_t)imax(bpg, 0), b = (uint32_t)deferred(sz, bpg), ta, tb;
+      block_scan2(a, b, ta, tb, wave_a, wave_b);
+      all += ta; cand += tb;
+    }
+    const long long live = (long long)imin((int32_t)all, U) * n_tiles;
+    const long long first = live / defer_cus * defer_cus;  // where the last round starts
+    defer_on = cand > 0 && (long long)(all - cand) * n_tiles >= first && (live - first) * 2 <= defer_slots && all <= (uint32_t)U;
+    total_regular = all - cand;
+  }
 
   for (int base = 0; base < g; base += kSchedThreads) {
     const int gi = base + tid;
     const int32_t sz = gi < g ? gs[gi] : 0;
-    const int32_t bpg = gi < g ? floor_div(sz + chunk - 1, chunk) : 0;  // gpu_ragged_dot.py:73
+    const int32_t bpg_all = gi < g ? floor_div(sz + chunk - 1, chunk) : 0;  // gpu_ragged_dot.py:73
+    const int32_t dfr = deferred(sz, bpg_all);
+    const int32_t bpg = bpg_all - dfr;  // tiles in the group's own run
     uint32_t a = (uint32_t)sz, b = (uint32_t)bpg, ta, tb;
     block_scan2(a, b, ta, tb, wave_a, wave_b);
     if (gi < g) group_offsets[gi] = (int32_t)(carry_rows + a - (uint32_t)sz);  // :86
     incl[tid] = (int32_t)(carry_tiles + b);
+    uint32_t td = 0;
+    if (defer_on) {
+      uint32_t c = (uint32_t)dfr, z = 0, tz;
+      block_scan2(c, z, td, tz, wave_a, wave_b);
+      incl_d[tid] = (int32_t)(carry_def + c);
+      tiles_of[tid] = bpg_all;
+    }
     __syncthreads();
 
     // Tiles [carry_tiles, carry_tiles + tb) belong to this slab of groups (:76-82).
@@ -96,10 +137,29 @@ __global__ __launch_bounds__(kSchedThreads) void sched_map_kernel(const int32_t*
         tile2band[t] = ((start + row0) << kBandShift) | rb;
       }
     }
+    // The deferred tiles of this slab of groups: slots total_regular + [carry_def, carry_def + td), each a band of its own.
+    if (defer_on) {
+      const int cnt_d = imin(kSchedThreads, g - base);
+      for (int32_t j = (int32_t)carry_def + tid; j < (int32_t)(carry_def + td); j += kSchedThreads) {
+        int l = 0, r = cnt_d;  // first group of the slab with incl_d > j
+        while (l < r) {
+          const int mid = (l + r) >> 1;
+          if (incl_d[mid] > j) r = mid; else l = mid + 1;
+        }
+        const int32_t slot = (int32_t)total_regular + j;
+        if (slot >= 0 && slot < U) {
+          tile2group[slot] = base + l;
+          tile2it[slot] = tiles_of[l] - 1;
+          if (tile2band) tile2band[slot] = kBandDeferred | (slot << kBandShift) | 1;
+        }
+      }
+    }
     carry_rows += ta;
     carry_tiles += tb;
+    carry_def += td;
     __syncthreads();
   }
+  carry_tiles += carry_def;  // all tiles
   // Unused slots read as zero (the masked sums of :81-82 are empty there).
   for (int32_t t = imax((int32_t)carry_tiles, 0) + tid; t < U; t += kSchedThreads) {
     tile2group[t] = 0;
@@ -110,7 +170,7 @@ __global__ __launch_bounds__(kSchedThreads) void sched_map_kernel(const int32_t*
 
   if (block_order) {
     // The blocks of the gmm tile walk, sorted into those of long groups (from the front) and the others (from the back);
-    // a block is judged by the group of its first position.
+    // a block is judged by its first position.
     __threadfence_block();
     __syncthreads();  // the map above is complete
     const int total = imax(imin((int32_t)carry_tiles, U), 0);
@@ -121,8 +181,9 @@ __global__ __launch_bounds__(kSchedThreads) void sched_map_kernel(const int32_t*
       const int b = base + tid;
       bool is_long = false, is_short = false;
       if (b < live_blocks) {
+        // (a long group's short last tile that was moved behind the others counts as short: it streams)
         const int slot = imin((int)(((long long)b * per_block) / n_tiles), total - 1);
-        is_long = gs[tile2group[slot]] > long_rows;
+        is_long = gs[tile2group[slot]] > long_rows && !(tile2band && (tile2band[slot] & kBandDeferred));
         is_short = !is_long;
       }
       uint32_t a = is_long, c = is_short, ta, tc;
@@ -217,14 +278,16 @@ int launch_stream_read(hipStream_t s, const void* src, size_t bytes, size_t bloc
 int launch_sched_map(hipStream_t s, const int32_t* gs, int g, int m, int chunk, int32_t* group_offsets,
                      int32_t* tile2group, int32_t* tile2it, int32_t* total_tiles, int32_t* counters, int n_counters,
                      int32_t* tile2band, int band_rows, int32_t* block_order, int n_blocks, int per_block, int n_tiles,
-                     int long_rows, int32_t* group_order, int order_first, int order_count) {
+                     int long_rows, int32_t* group_order, int order_first, int order_count, int defer_rows,
+                     int defer_cus, int defer_slots) {
   const int U = (m + chunk - 1) / chunk + g;  // gpu_ragged_dot.py:77
   if (band_rows < 1) band_rows = 1;
   if (band_rows > kBandMaxRows) band_rows = kBandMaxRows;
   hipLaunchKernelGGL(sched_map_kernel, dim3(1), dim3(kSchedThreads), 0, s, gs, g, U, chunk, group_offsets,
                      tile2group, tile2it, total_tiles, counters, counters ? n_counters : 0, tile2band, band_rows,
                      n_blocks > 0 ? block_order : nullptr, n_blocks, per_block > 0 ? per_block : 1, n_tiles > 0 ? n_tiles : 1,
-                     long_rows, order_count > 0 ? group_order : nullptr, order_first, order_count);
+                     long_rows, order_count > 0 ? group_order : nullptr, order_first, order_count, tile2band ? defer_rows : 0, defer_cus,
+                     defer_slots);
   return (int)hipGetLastError();
 }
 

@@ -319,6 +319,70 @@ def test_k_split_of_last_round(vid, vname, shape, trans_rhs):
     assert np.array_equal(util.to_np(y).astype(np.float32), -2.0 * outs[0].astype(np.float32))
 
 
+@pytest.mark.parametrize("trans_rhs", [False, True], ids=["A", "At"])
+@pytest.mark.parametrize("case", ["plan_cut", "long_k", "too_many"])
+def test_short_last_tiles_move_into_the_k_split_round(case, trans_rhs):
+    """Four-wave 256 x 256 core with the last round of tiles cut along K: the last row tile of a group of several row
+    tiles, when it holds at most 128 rows, is listed behind all other tiles (marked in the band array of the internal
+    map) and runs through the streaming routines - if all such tiles then lie in that last round.  Same bounds against
+    the oracle, every element written, the same bits on a second call; without the K-split nothing moves."""
+    print(f"short last tiles {case} trans_rhs {trans_rhs}", flush=True)
+    if case == "plan_cut":  # cut by the plan (k itself would not ask for it)
+        k, n, lens, split_k = 1096, 520, [300, 0, 520, 356, 700, 90], 8
+        moved = [(0, 1), (2, 2), (3, 1)]
+    elif case == "long_k":  # cut because k is long
+        k, n, lens, split_k = 6664, 256, [600, 290, 0, 128], 0
+        moved = [(0, 2), (1, 1)]
+    else:  # 280 tiles, a round of 256 and a last one of 24: the 140 short last tiles would not all lie in the last one
+        k, n, lens, split_k = 1032, 512, [260 + i for i in range(70)], 8
+        moved = []
+    rng = np.random.default_rng(31)
+    gs = np.array(lens, np.int32)
+    g = len(lens)
+    rows = int(gs.sum())
+    m = rows + 13
+    lhs = oracle.round_to(rng.standard_normal((m, k)).astype(np.float32), "bfloat16")
+    rhs = oracle.round_to((rng.standard_normal((g, k, n)) / k ** 0.5).astype(np.float32), "bfloat16")
+    x = util.bf16_dev(lhs)
+    A = util.bf16_dev(np.ascontiguousarray(np.swapaxes(rhs, 1, 2)) if trans_rhs else rhs)
+    gs_d = torch.from_numpy(gs).cuda()
+    vid = [v.id for v in _capi.variants() if v.name.decode() == "w256x256x32_w2x2_s5"][0]
+    split, whole = _capi.Plan(vid, 2, 0, 4, split_k=split_k), _capi.Plan(vid, 2, 0, 4, split_k=-1)
+    need = _capi.lib.rd_gmm_workspace_bytes(m, g, ctypes.byref(split))
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    U = -(-m // 256) + g
+    n_all = int(np.sum(-(-gs // 256)))
+    outs, maps = [], []
+    for plan in (split, split, whole):
+        ws.fill_(0xA5)
+        y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        rc = _capi.lib.rd_gmm(torch.cuda.current_stream().cuda_stream, x.data_ptr(), A.data_ptr(), gs_d.data_ptr(),
+                              y.data_ptr(), m, k, n, g, int(trans_rhs), _capi.RD_DTYPE_BF16, ctypes.byref(plan),
+                              ws.data_ptr(), ws.numel())
+        torch.cuda.synchronize()
+        assert rc == 0, _capi.lib.rd_last_error()
+        outs.append(util.to_np(y))
+        w = ws.view(torch.int32).cpu().numpy()
+        maps.append((w[g:g + U].copy(), w[g + U:g + 2 * U].copy(), w[g + 2 * U + 1:g + 3 * U + 1].copy()))
+    y_ref = oracle.gmm(lhs, rhs, gs)
+    for y in outs:
+        assert not np.isnan(y).any()
+        util.assert_close_rows(y, y_ref, rows, util.BF16_EPS, "y")
+        assert not np.any(y[rows:])
+    assert np.array_equal(outs[0], outs[1])
+    mark = 1 << 30
+    group_of, tile_of, band = maps[0]
+    assert int(np.count_nonzero(band[:n_all] & mark)) == len(moved)
+    if moved:
+        assert [(int(a), int(b)) for a, b in zip(group_of[n_all - len(moved):n_all], tile_of[n_all - len(moved):n_all])] == moved
+        assert not np.any(band[:n_all - len(moved)] & mark)
+    # every (group, row tile) pair is listed once, moved or not
+    want = sorted((gi, it) for gi in range(g) for it in range(-(-int(gs[gi]) // 256)))
+    assert sorted(zip(group_of[:n_all].tolist(), tile_of[:n_all].tolist())) == want
+    assert not np.any(maps[2][2][:n_all] & mark)
+    assert list(zip(maps[2][0][:n_all].tolist(), maps[2][1][:n_all].tolist())) == want
+
+
 # ---------------------------------------------------------------------------------------------------------------------
 # configuration C1 (tiny) with its exact recipe, and the other configurations' shapes
 # ---------------------------------------------------------------------------------------------------------------------
