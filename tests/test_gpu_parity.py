@@ -320,7 +320,7 @@ def test_k_split_of_last_round(vid, vname, shape, trans_rhs):
 
 
 @pytest.mark.parametrize("trans_rhs", [False, True], ids=["A", "At"])
-@pytest.mark.parametrize("case", ["plan_cut", "long_k", "too_many"])
+@pytest.mark.parametrize("case", ["plan_cut", "long_k", "too_many", "many_groups"])
 def test_short_last_tiles_move_into_the_k_split_round(case, trans_rhs):
     """Four-wave 256 x 256 core with the last round of tiles cut along K: the last row tile of a group of several row
     tiles, when it holds at most 128 rows, is listed behind all other tiles (marked in the band array of the internal
@@ -333,6 +333,12 @@ def test_short_last_tiles_move_into_the_k_split_round(case, trans_rhs):
     elif case == "long_k":  # cut because k is long
         k, n, lens, split_k = 6664, 256, [600, 290, 0, 128], 0
         moved = [(0, 2), (1, 1)]
+    elif case == "many_groups":  # more groups than the map kernel scans at a time, moved tiles in its second pass
+        k, n, split_k = 1032, 128, 8
+        lens = [0] * 1100
+        for gi, rows in ((5, 300), (17, 64), (600, 256), (1030, 520), (1031, 128), (1090, 290), (1099, 1)):
+            lens[gi] = rows
+        moved = [(5, 1), (1030, 2), (1090, 1)]
     else:  # 280 tiles, a round of 256 and a last one of 24: the 140 short last tiles would not all lie in the last one
         k, n, lens, split_k = 1032, 512, [260 + i for i in range(70)], 8
         moved = []
