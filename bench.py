@@ -370,7 +370,7 @@ def schedule_context(torch):
     this process: gmm trans_rhs (dlhs) with the blocks of long and short groups dealt interleaved (what a call with the
     full workspace does) against the walk order (the same call through the C ABI with a workspace that holds only the
     scheduling map); tgmm (drhs) with the groups visited by falling size class (plan group_n = 1, the tuned plan) against
-    the order they come in (group_n = 0)."""
+    the order they come in (group_n = -1)."""
     import ctypes
 
     from gpu_ragged_dot_amd import _capi, ops, planner, workloads
@@ -396,7 +396,7 @@ def schedule_context(torch):
             fn()
         out[label] = _event_ms(fn, 20, torch)
     tuned = planner.select_plan(_capi.OP_TGMM, m, k, n, g)
-    for label, gn in (("drhs_groups_by_size_class", 1), ("drhs_groups_as_they_come", 0)):
+    for label, gn in (("drhs_groups_by_size_class", 1), ("drhs_groups_as_they_come", -1)):
         p2 = _capi.Plan(tuned.variant, tuned.group_m, 0, gn, 0)
         fn = lambda: ops._tgmm_fwd(x, dout, gs, **HP, acc_dtype=torch.float32, plan=p2)
         for _ in range(3):

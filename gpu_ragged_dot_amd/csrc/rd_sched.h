@@ -27,7 +27,7 @@ constexpr int kBandDeferred = 1 << 30;  // mark of a short last row tile listed 
 // by side (DeepSeek-V3 shape, 256 groups of 0 to 7099 rows: 1.97 -> 1.92 ms; with the groups also stored in that order
 // 1.90; an exact sort by rows gives the same, classes of 64 or 128 rows half of it or nothing, long groups merely moved
 // to the front nothing).  Where two groups' tiles share an XCD the order the groups come in mixes long and short
-// tiles and is the better one (128 groups with Zipf lengths, k 2048, n 4096: 0.84 -> 0.88 ms), hence an option of the plan.
+// tiles and is the better one (128 groups with Zipf lengths, k 2048, n 4096: 0.84 -> 0.88 ms), so the caller of this function decides.
 // `defer_rows` > 0 (internal maps of gmm launches only, needs tile2band): the last row tile of a group of two or more
 // row tiles, when it holds at most defer_rows rows, is listed behind all other tiles instead of behind its group's - as a
 // band of its own, marked kBandDeferred - provided all such tiles then lie in the launch's partly filled last round

@@ -50,8 +50,8 @@ def sweep(x, A, dout, gs, op: int, reps: int = 10, rounds: int = 3):
     n = A.shape[2]
     vec = k % 8 == 0 and n % 8 == 0
     # gmm: (most row tiles per band, columns per block); the product is what one XCD is dealt at a time, 32 tiles suit
-    # one work-group per compute unit.  tgmm: (row tiles per band, 1 = groups visited by falling size class).
-    walks = [(0, 0), (1, 32), (2, 16), (4, 8), (8, 4), (2, 4), (4, 4)] if op != _capi.OP_TGMM else [(1, 0), (2, 0), (4, 0), (8, 0), (16, 0), (4, 1), (8, 1)]
+    # one work-group per compute unit.  tgmm: (row tiles per band, 1 = groups visited by falling size class, -1 = as they come).
+    walks = [(0, 0), (1, 32), (2, 16), (4, 8), (8, 4), (2, 4), (4, 4)] if op != _capi.OP_TGMM else [(1, -1), (2, -1), (4, -1), (8, -1), (16, -1), (4, 1), (8, 1)]
     cands = []
     for v in planner.compiled_variants():
         if bool(v.vec) != vec or v.dtype != _capi.RD_DTYPE_BF16:

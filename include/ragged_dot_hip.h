@@ -81,7 +81,8 @@ typedef struct rd_plan {
   int group_n; /* rd_gmm: the walk is dealt to the 8 XCDs in blocks of group_m x group_n (<= 4096) consecutive tiles;
                   the product should equal what one XCD runs at a time (32 for the 256 x 256 tiles).  0 = default.
                   rd_tgmm: 1 = visit the groups by falling row count class (tiles of about equal duration then run side
-                  by side; worth trying when one group's tiles fill most of an XCD), anything else = as they come */
+                  by side, and the longest groups' tiles do not end the launch alone), -1 = as they come, 0 = by size
+                  class when the groups average 512 rows or more and the launch has more than a round of tiles */
   int decode_nb; /* rd_gmm only, for a few rows per group: > 0 selects the streaming kernel that gives each work-group
                     this many columns (32, 64 or 128) of one expert; RD_DECODE_ROWS the one that gives it whole rows
                     for a slice of the contraction range (fp32 partial sums in the workspace, n <= 2048) or, with
@@ -166,7 +167,7 @@ int rd_gmm_noalloc(void* stream, const void* x, const void* A, const int32_t* gr
  * Replaces the "gpu_tgmm" pallas_call (gpu_ragged_dot.py:231-281, 331-340).  Slices of empty groups are zero
  * (:277-281).  x is [m, k], dy is [m, n].
  * Workspace: rd_tgmm_workspace_bytes() bytes, 256-byte aligned: the groups' row offsets and 16 bytes per group for the
- * order in which the launch visits the groups when the plan asks for one (group_n = 1).  A workspace with room for the
+ * order in which the launch visits the groups when they go by size class (group_n of the plan).  A workspace with room for the
  * offsets only is accepted: the groups are then visited as they come - same results. */
 size_t rd_tgmm_workspace_bytes(int m, int g, const rd_plan* plan /* host, may be NULL */);
 int rd_tgmm(void* stream, const void* x, const void* dy, const int32_t* group_sizes, void* dA, int m, int k,

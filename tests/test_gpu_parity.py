@@ -224,6 +224,45 @@ def test_tgmm_group_order_is_transparent(vname, g_first, g_local):
     assert not np.any(got[gs[sl] == 0])
 
 
+@pytest.mark.parametrize("vname", [None, "d128x128x32_w2x2_s3", "w256x256x32_w2x2_s5"])
+def test_tgmm_group_order_by_default_for_long_groups(vname):
+    """plan.group_n = 0 leaves the order of the groups to the library: by size class when the groups average 512 rows
+    or more, the launch has more than a round of tiles and the product is not tiny; -1 keeps the order they come in.
+    Same tiles either way: equal bits, and the order records in the workspace are written only in the first case."""
+    print(f"tgmm default group order {vname}", flush=True)
+    k, n = 2048, 2304
+    gs = np.array([900, 150, 0, 1400, 610], np.int32)
+    g = len(gs)
+    m = int(gs.sum()) + 12
+    assert m >= 512 * g and m * k * n >= 8e9
+    rng = np.random.default_rng(29)
+    lhs = oracle.round_to(rng.standard_normal((m, k)).astype(np.float32), "bfloat16")
+    dout = oracle.round_to(rng.standard_normal((m, n)).astype(np.float32), "bfloat16")
+    vid = -1 if vname is None else [v.id for v in _capi.variants() if v.name.decode() == vname][0]
+    x, d, gsd = util.bf16_dev(lhs), util.bf16_dev(dout), torch.from_numpy(gs).cuda()
+    offsets_only = -(-((g + 3 * (g + 1) + 1) * 4) // 256) * 256
+    stream = torch.cuda.current_stream().cuda_stream
+    outs, touched = [], []
+    for group_n in (0, -1, 1):
+        plan = _capi.Plan(vid, 0, 0, group_n)
+        ws_bytes = _capi.lib.rd_tgmm_workspace_bytes(m, g, ctypes.byref(plan))
+        assert ws_bytes >= offsets_only + 16 * g
+        ws = torch.full((ws_bytes,), 0xA5, dtype=torch.uint8, device="cuda")
+        dA = torch.full((g, k, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        rc = _capi.lib.rd_tgmm(stream, x.data_ptr(), d.data_ptr(), gsd.data_ptr(), dA.data_ptr(), m, k, n, g,
+                               _capi.RD_DTYPE_BF16, ctypes.byref(plan), ws.data_ptr(), ws_bytes)
+        assert rc == _capi.RD_OK, _capi.lib.rd_last_error()
+        torch.cuda.synchronize()
+        outs.append(dA)
+        touched.append(bool((ws[offsets_only:offsets_only + 16 * g] != 0xA5).any().item()))
+    assert touched == [True, False, True]
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+    assert torch.equal(outs[0].view(torch.int16), outs[2].view(torch.int16))
+    got = util.to_np(outs[0])
+    util.assert_close_groups(got, oracle.tgmm(lhs, dout, gs), gs != 0, util.TGMM_BF16_EPS, "tgmm default group order")
+    assert not np.any(got[gs == 0])
+
+
 @pytest.mark.parametrize("trans_rhs", [False, True], ids=["A", "At"])
 @pytest.mark.parametrize("vname,walk", [("w256x256x32_w2x2_s5", (4, 8)), ("w256x256x32_w2x2_s5", (2, 4)),
                                         ("p256x256x32_w2x4_s4", (3, 5)), ("d128x128x32_w2x2_s3", (4, 8))])
