@@ -167,7 +167,11 @@ def measure(name, steps, warmup, torch, sustained_seconds=0.0, headline=False):
     if len(parts) == 1:  # the step is that one product: the timed region already is its launch duration
         per = {parts[0][0]: ms_per_step}
     else:
-        per = {pname: _event_ms(fn, max(steps, 5), torch) for pname, fn in parts}
+        per = {}
+        for pname, fn in parts:
+            for _ in range(2):  # the other products ran last: let this one's operands and code settle first
+                fn()
+            per[pname] = _event_ms(fn, max(steps, 5), torch)
     dominant = max(per, key=per.get)
     flops_step = workloads.flops(name)
     abytes = workloads.algorithmic_bytes(name)
