@@ -166,6 +166,12 @@ def test_default_plan_scales_the_tile_with_the_problem():
     assert tile(_capi.OP_GMM_TRANS, 1536, 8192, 1024, 3) == (128, 128)   # ... but not with a contraction of 8192
     # trans_rhs, long contraction, under a round of 256 x 256 tiles: the eight-wave 256 x 256 core and its K-split
     assert vs[_capi.default_plan(_capi.OP_GMM_TRANS, 512, 8192, 8192, 1).variant].name.decode() == "p256x256x32_w2x4_s4"
+    name = lambda op, m, k, n, g: vs[_capi.default_plan(op, m, k, n, g).variant].name.decode()
+    # forward product, few tiles: the four-wave core for long groups, the eight-wave per-operand-ring one for groups of a tile's height
+    assert name(_capi.OP_GMM, 6144, 6144, 1536, 6) == "w256x256x32_w2x2_s5" and name(_capi.OP_GMM, 1792, 7168, 7168, 7) == "q256x256x32_w2x4"
+    # tgmm with groups far shorter than a tile: three 128 x 128 work-groups per compute unit (not at the DeepSeek-V3 size)
+    assert tile(_capi.OP_TGMM, 3072, 3072, 3072, 48) == (128, 128) and tile(_capi.OP_TGMM, 4096, 7168, 2048, 64) == (128, 128)
+    assert tile(_capi.OP_TGMM, 16384, 2048, 4096, 128) == (256, 256)
     assert tile(_capi.OP_GMM, 8192, 4096, 4096, 8, dtype=_capi.RD_DTYPE_F32) == (128, 128)
     assert tile(_capi.OP_GMM, 512, 256, 256, 4, dtype=_capi.RD_DTYPE_F32) == (64, 64)
 
