@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-/* 3: RD_DTYPE_F16; rd_plan.group_n = 1 for rd_tgmm; the workspaces hold the orders the scheduling-map kernel builds
+/* 3: RD_DTYPE_F16; rd_plan.group_n = 1 / -1 for rd_tgmm; the workspaces hold the orders the scheduling-map kernel builds
  * (all source compatible with 2: same structs, same signatures) */
 #define RD_ABI_VERSION 3
 
